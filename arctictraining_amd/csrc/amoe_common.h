@@ -1,0 +1,147 @@
+// Shared host/device helpers for the gfx950 expert-layer kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/arctic_moe_hip.h"
+
+#define AMOE_EXPORT extern "C" __attribute__((visibility("default")))
+
+// ---------------------------------------------------------------- host side errors
+void amoe_set_error(const char* fmt, ...);
+
+#define AMOE_REQUIRE(cond, code, ...)  \
+    do {                               \
+        if (!(cond)) {                 \
+            amoe_set_error(__VA_ARGS__); \
+            return (code);             \
+        }                              \
+    } while (0)
+
+static inline int amoe_check_launch(const char* what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        amoe_set_error("%s: %s", what, hipGetErrorString(e));
+        return AMOE_ERR_LAUNCH;
+    }
+    return AMOE_OK;
+}
+
+// ---------------------------------------------------------------- device types
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+#define AMOE_WAVE 64
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t hi16) { return __uint_as_float(hi16 << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// round-to-nearest-even float -> bf16 pair packed into one dword (lo = a, hi = b)
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b)
+{
+    f32x2_t v = {a, b};
+    bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ float round_bf16(float a)
+{
+    bf16_t r = (bf16_t)a;
+    return (float)r;
+}
+
+template <typename T>
+struct ElemTraits;
+template <>
+struct ElemTraits<float> {
+    static constexpr int kVec = 4;  // elements per 16-byte vector
+    __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(v[i]);
+    }
+    __device__ static __forceinline__ u32x4_t pack(const float* f)
+    {
+        u32x4_t v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __float_as_uint(f[i]);
+        return v;
+    }
+    __device__ static __forceinline__ float load1(const float* p) { return *p; }
+    __device__ static __forceinline__ void store1(float* p, float v) { *p = v; }
+    __device__ static __forceinline__ float round(float v) { return v; }
+};
+template <>
+struct ElemTraits<bf16_t> {
+    static constexpr int kVec = 8;
+    __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = bf16_lo(v[i]);
+            f[2 * i + 1] = bf16_hi(v[i]);
+        }
+    }
+    __device__ static __forceinline__ u32x4_t pack(const float* f)
+    {
+        u32x4_t v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = pack_bf16x2(f[2 * i], f[2 * i + 1]);
+        return v;
+    }
+    __device__ static __forceinline__ float load1(const bf16_t* p) { return (float)(*p); }
+    __device__ static __forceinline__ void store1(bf16_t* p, float v) { *p = (bf16_t)v; }
+    __device__ static __forceinline__ float round(float v) { return round_bf16(v); }
+};
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, AMOE_WAVE);
+    return v;
+}
+
+// activations of the gated expert FFN (value and derivative)
+template <int ACT>
+__device__ __forceinline__ float act_fwd(float g)
+{
+    if (ACT == AMOE_ACT_SILU) return g / (1.0f + __expf(-g));
+    if (ACT == AMOE_ACT_GPT_OSS) return g / (1.0f + __expf(-1.702f * g));
+    if (ACT == AMOE_ACT_RELU) return g > 0.f ? g : 0.f;
+    // exact (erf) gelu, the default of torch.nn.functional.gelu
+    return 0.5f * g * (1.0f + erff(g * 0.70710678118654752f));
+}
+template <int ACT>
+__device__ __forceinline__ float act_bwd(float g)
+{
+    if (ACT == AMOE_ACT_SILU) {
+        float s = 1.0f / (1.0f + __expf(-g));
+        return s * (1.0f + g * (1.0f - s));
+    }
+    if (ACT == AMOE_ACT_GPT_OSS) {
+        float s = 1.0f / (1.0f + __expf(-1.702f * g));
+        return s * (1.0f + 1.702f * g * (1.0f - s));
+    }
+    if (ACT == AMOE_ACT_RELU) return g > 0.f ? 1.f : 0.f;
+    float cdf = 0.5f * (1.0f + erff(g * 0.70710678118654752f));
+    float pdf = 0.3989422804014327f * __expf(-0.5f * g * g);
+    return cdf + g * pdf;
+}
+
+#define AMOE_DISPATCH_ACT(act, ...)                                  \
+    switch (act) {                                                   \
+        case AMOE_ACT_SILU: { constexpr int ACT = AMOE_ACT_SILU; __VA_ARGS__; } break;       \
+        case AMOE_ACT_GELU: { constexpr int ACT = AMOE_ACT_GELU; __VA_ARGS__; } break;       \
+        case AMOE_ACT_RELU: { constexpr int ACT = AMOE_ACT_RELU; __VA_ARGS__; } break;       \
+        default: { constexpr int ACT = AMOE_ACT_GPT_OSS; __VA_ARGS__; } break;               \
+    }

@@ -1,0 +1,147 @@
+// Exported grouped-GEMM entry points (argument validation + dtype dispatch), the version
+// query and the per-thread error message.
+#include "amoe_common.h"
+
+#include <string.h>
+
+static thread_local char g_err[512] = "";
+
+void amoe_set_error(const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+AMOE_EXPORT int amoe_version(void) { return 100; }
+AMOE_EXPORT const char* amoe_last_error(void) { return g_err; }
+
+// implemented in gemm_bf16.hip / gemm_f32.hip / rows.hip
+int amoe_bf16_gateup_act(const void* xp, const int32_t* a_row_map, const void* w, const int32_t* offsets, void* gate_up,
+                         void* inter, int R, int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
+                         int tile_cfg, hipStream_t s);
+int amoe_bf16_nn(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
+                 int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s);
+int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
+                 int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s);
+int amoe_bf16_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int R, int E, int Kd, int N,
+                    int tile_cfg, hipStream_t s);
+int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
+                  int Kred, int N, int ldb, long long strideB, bool b_kc, void* workspace, size_t workspace_bytes,
+                  hipStream_t s);
+int amoe_f32_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int R, int E, int Kd, int N,
+                   hipStream_t s);
+int amoe_launch_gated_act_fwd(const void* gu, void* inter, int dtype, int R, int I, int act, hipStream_t s);
+
+namespace {
+
+// what both dtypes share: pointers, sizes, the int32 offset range
+int check_gemm_common(const char* what, int dtype, int R, int E, int d0, int d1, int tile_cfg)
+{
+    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "%s: bad dtype %d", what, dtype);
+    AMOE_REQUIRE(R > 0 && E > 0 && d0 > 0 && d1 > 0, AMOE_ERR_BAD_ARG, "%s: sizes must be positive (R=%d E=%d %d %d)",
+                 what, R, E, d0, d1);
+    AMOE_REQUIRE(E <= AMOE_MAX_EXPERTS, AMOE_ERR_UNSUPPORTED, "%s: E=%d exceeds %d", what, E, AMOE_MAX_EXPERTS);
+    AMOE_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, AMOE_ERR_BAD_ARG, "%s: tile_cfg %d outside 0..3", what, tile_cfg);
+    AMOE_REQUIRE((long long)R * d0 < (1ll << 32) && (long long)R * d1 < (1ll << 32) && (long long)d0 * d1 < (1ll << 32),
+                 AMOE_ERR_UNSUPPORTED, "%s: an operand exceeds 2^32 elements", what);
+    return AMOE_OK;
+}
+
+// reduction length must be a multiple of `red_mult`, the other extents of `vec`
+int check_gemm_dims(const char* what, int dtype, int red, int other)
+{
+    if (dtype == AMOE_BF16) {
+        AMOE_REQUIRE(red % 64 == 0, AMOE_ERR_UNSUPPORTED, "%s: bf16 reduction length %d must be a multiple of 64", what,
+                     red);
+        AMOE_REQUIRE(other % 8 == 0, AMOE_ERR_UNSUPPORTED, "%s: bf16 extent %d must be a multiple of 8", what, other);
+    } else {
+        AMOE_REQUIRE(red % 4 == 0 && other % 4 == 0, AMOE_ERR_UNSUPPORTED,
+                     "%s: f32 extents (%d, %d) must be multiples of 4", what, red, other);
+    }
+    return AMOE_OK;
+}
+
+}  // namespace
+
+AMOE_EXPORT int amoe_grouped_gemm_gateup_act_fwd(const void* xp, const int32_t* a_row_map, const void* w_gate_up,
+                                                 const int32_t* offsets, void* gate_up, void* inter, int dtype, int R,
+                                                 int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
+                                                 int tile_cfg, void* stream)
+{
+    const char* what = "grouped_gemm_gateup_act_fwd";
+    AMOE_REQUIRE(xp && w_gate_up && offsets && inter && workspace, AMOE_ERR_BAD_ARG, "%s: null pointer", what);
+    int rc = check_gemm_common(what, dtype, R, E, H, I, tile_cfg);
+    if (rc) return rc;
+    AMOE_REQUIRE(act >= AMOE_ACT_SILU && act <= AMOE_ACT_GPT_OSS, AMOE_ERR_BAD_ARG, "%s: bad activation %d", what, act);
+    AMOE_REQUIRE((long long)H * 2 * I < (1ll << 32) && (long long)R * 2 * I < (1ll << 32), AMOE_ERR_UNSUPPORTED,
+                 "%s: an operand exceeds 2^32 elements", what);
+    rc = check_gemm_dims(what, dtype, H, 2 * I);
+    if (rc) return rc;
+    AMOE_REQUIRE(workspace_bytes >= amoe_grouped_gemm_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
+                 "%s: workspace %zu < %zu bytes", what, workspace_bytes, amoe_grouped_gemm_workspace_bytes(R, E));
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == AMOE_BF16)
+        return amoe_bf16_gateup_act(xp, a_row_map, w_gate_up, offsets, gate_up, inter, R, E, H, I, act, workspace,
+                                    workspace_bytes, tile_cfg, s);
+    AMOE_REQUIRE(gate_up, AMOE_ERR_UNSUPPORTED, "%s: the f32 path needs the gate_up buffer", what);
+    AMOE_REQUIRE(I % 4 == 0, AMOE_ERR_UNSUPPORTED, "%s: f32 intermediate size %d must be a multiple of 4", what, I);
+    rc = amoe_f32_rows(xp, a_row_map, w_gate_up, offsets, gate_up, R, E, H, 2 * I, 2 * I, (long long)H * 2 * I, false,
+                       workspace, workspace_bytes, s);
+    if (rc) return rc;
+    return amoe_launch_gated_act_fwd(gate_up, inter, dtype, R, I, act, s);
+}
+
+AMOE_EXPORT int amoe_grouped_gemm_nn(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets,
+                                     void* C, int dtype, int R, int E, int Kd, int N, void* workspace,
+                                     size_t workspace_bytes, int tile_cfg, void* stream)
+{
+    const char* what = "grouped_gemm_nn";
+    AMOE_REQUIRE(A && B && offsets && C && workspace, AMOE_ERR_BAD_ARG, "%s: null pointer", what);
+    int rc = check_gemm_common(what, dtype, R, E, Kd, N, tile_cfg);
+    if (rc) return rc;
+    rc = check_gemm_dims(what, dtype, Kd, N);
+    if (rc) return rc;
+    AMOE_REQUIRE(workspace_bytes >= amoe_grouped_gemm_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
+                 "%s: workspace %zu < %zu bytes", what, workspace_bytes, amoe_grouped_gemm_workspace_bytes(R, E));
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == AMOE_BF16)
+        return amoe_bf16_nn(A, a_row_map, B, offsets, C, R, E, Kd, N, workspace, workspace_bytes, tile_cfg, s);
+    return amoe_f32_rows(A, a_row_map, B, offsets, C, R, E, Kd, N, N, (long long)Kd * N, false, workspace,
+                         workspace_bytes, s);
+}
+
+AMOE_EXPORT int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets,
+                                     void* C, int dtype, int R, int E, int Kd, int N, void* workspace,
+                                     size_t workspace_bytes, int tile_cfg, void* stream)
+{
+    const char* what = "grouped_gemm_nt";
+    AMOE_REQUIRE(A && B && offsets && C && workspace, AMOE_ERR_BAD_ARG, "%s: null pointer", what);
+    int rc = check_gemm_common(what, dtype, R, E, Kd, N, tile_cfg);
+    if (rc) return rc;
+    rc = check_gemm_dims(what, dtype, N, Kd);  // the reduction runs over N here
+    if (rc) return rc;
+    AMOE_REQUIRE(workspace_bytes >= amoe_grouped_gemm_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
+                 "%s: workspace %zu < %zu bytes", what, workspace_bytes, amoe_grouped_gemm_workspace_bytes(R, E));
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == AMOE_BF16)
+        return amoe_bf16_nt(A, a_row_map, B, offsets, C, R, E, Kd, N, workspace, workspace_bytes, tile_cfg, s);
+    return amoe_f32_rows(A, a_row_map, B, offsets, C, R, E, /*Kred=*/N, /*N out=*/Kd, /*ldb=*/N, (long long)Kd * N, true,
+                         workspace, workspace_bytes, s);
+}
+
+AMOE_EXPORT int amoe_grouped_gemm_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int dtype, int R,
+                                        int E, int Kd, int N, int tile_cfg, void* stream)
+{
+    const char* what = "grouped_gemm_wgrad";
+    AMOE_REQUIRE(A && B && offsets && C, AMOE_ERR_BAD_ARG, "%s: null pointer", what);
+    int rc = check_gemm_common(what, dtype, R, E, Kd, N, tile_cfg);
+    if (rc) return rc;
+    const int vec = dtype == AMOE_BF16 ? 8 : 4;
+    AMOE_REQUIRE(Kd % vec == 0 && N % vec == 0, AMOE_ERR_UNSUPPORTED, "%s: extents (%d, %d) must be multiples of %d",
+                 what, Kd, N, vec);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == AMOE_BF16) return amoe_bf16_wgrad(A, B, offsets, C, R, E, Kd, N, tile_cfg, s);
+    return amoe_f32_wgrad(A, B, offsets, C, R, E, Kd, N, s);
+}

@@ -1,0 +1,146 @@
+// Deterministic token-to-expert permutation plan: a stable counting sort of the k-major
+// flattened assignment vector, in three launches
+//   1. per-chunk expert histograms (LDS counters),
+//   2. a one-block scan over chunks and experts (counts, offsets, per-chunk bases),
+//   3. per-chunk ranking in ascending slot order (ballot match inside a wavefront, LDS
+//      running counters across steps) and the scatter of the three index maps.
+// A chunk is kChunk consecutive flat slots f = k*T + t handled by ONE wavefront, so the
+// order inside an expert is ascending f by construction, with no global atomics.
+#include "amoe_common.h"
+
+namespace {
+
+constexpr int kChunk = 1024;        // flat slots per wavefront
+constexpr int kWavesPerBlock = 4;   // independent chunks per block
+
+__device__ __forceinline__ int load_expert(const int32_t* assign, int f, int T, int K, int E)
+{
+    int k = f / T;
+    int t = f - k * T;
+    int e = assign[(size_t)t * K + k];
+    return min(max(e, 0), E - 1);  // memory safety for caller-supplied assignments
+}
+
+__global__ void __launch_bounds__(kWavesPerBlock * AMOE_WAVE)
+permute_hist_kernel(const int32_t* __restrict__ assign, int T, int K, int E, int R, int n_chunks,
+                    int32_t* __restrict__ chunk_counts)
+{
+    __shared__ int32_t cnt[kWavesPerBlock][AMOE_MAX_EXPERTS];
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c = blockIdx.x * kWavesPerBlock + w;
+    for (int e = lane; e < E; e += 64) cnt[w][e] = 0;
+    __syncthreads();
+    if (c < n_chunks) {
+        const int f0 = c * kChunk;
+        const int f1 = min(f0 + kChunk, R);
+        for (int f = f0 + lane; f < f1; f += 64) atomicAdd(&cnt[w][load_expert(assign, f, T, K, E)], 1);
+    }
+    __syncthreads();
+    if (c < n_chunks)
+        for (int e = lane; e < E; e += 64) chunk_counts[(size_t)c * E + e] = cnt[w][e];
+}
+
+// one block of 512 threads: thread e owns expert e
+__global__ void __launch_bounds__(AMOE_MAX_EXPERTS)
+permute_scan_kernel(int32_t* __restrict__ chunk_counts /* in: counts, out: exclusive base inside expert */,
+                    int E, int n_chunks, int32_t* __restrict__ counts, int32_t* __restrict__ offsets)
+{
+    __shared__ int32_t tot[AMOE_MAX_EXPERTS];
+    const int e = threadIdx.x;
+    int run = 0;
+    if (e < E) {
+        for (int c = 0; c < n_chunks; ++c) {
+            int v = chunk_counts[(size_t)c * E + e];
+            chunk_counts[(size_t)c * E + e] = run;
+            run += v;
+        }
+        counts[e] = run;
+    }
+    tot[e] = (e < E) ? run : 0;
+    __syncthreads();
+    // Hillis-Steele inclusive scan over experts
+    for (int o = 1; o < AMOE_MAX_EXPERTS; o <<= 1) {
+        int add = (e >= o) ? tot[e - o] : 0;
+        __syncthreads();
+        tot[e] += add;
+        __syncthreads();
+    }
+    if (e < E) offsets[e + 1] = tot[e];
+    if (e == 0) offsets[0] = 0;
+}
+
+__global__ void __launch_bounds__(kWavesPerBlock * AMOE_WAVE)
+permute_scatter_kernel(const int32_t* __restrict__ assign, int T, int K, int E, int R, int n_chunks,
+                       const int32_t* __restrict__ chunk_base, const int32_t* __restrict__ offsets,
+                       int32_t* __restrict__ token_of, int32_t* __restrict__ slot_of, int32_t* __restrict__ row_of)
+{
+    __shared__ int32_t run[kWavesPerBlock][AMOE_MAX_EXPERTS];
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c = blockIdx.x * kWavesPerBlock + w;
+    if (c >= n_chunks) return;  // no block-wide barrier below: every wavefront is independent
+    for (int e = lane; e < E; e += 64) run[w][e] = offsets[e] + chunk_base[(size_t)c * E + e];
+    __builtin_amdgcn_wave_barrier();
+    const int f0 = c * kChunk;
+    const int f1 = min(f0 + kChunk, R);
+    const unsigned long long lt_mask = (1ull << lane) - 1ull;
+    for (int fb = f0; fb < f1; fb += 64) {
+        const int f = fb + lane;
+        const bool valid = f < f1;
+        const int e = valid ? load_expert(assign, f, T, K, E) : 0;
+        // lanes that hold the same expert
+        unsigned long long same = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 9; ++b) {
+            unsigned long long bits = __ballot((e >> b) & 1);
+            same &= ((e >> b) & 1) ? bits : ~bits;
+        }
+        const int rank = __popcll(same & lt_mask);
+        int row = 0;
+        if (valid) row = run[w][e] + rank;
+        __builtin_amdgcn_wave_barrier();
+        // the highest lane of each group advances the running counter
+        if (valid && (same >> lane) == 1ull) run[w][e] = row + 1;
+        __builtin_amdgcn_wave_barrier();
+        if (valid) {
+            int k = f / T;
+            int t = f - k * T;
+            token_of[row] = t;
+            slot_of[row] = f;
+            row_of[(size_t)t * K + k] = row;
+        }
+    }
+}
+
+}  // namespace
+
+static inline int permute_chunks(int R) { return (R + kChunk - 1) / kChunk; }
+
+AMOE_EXPORT size_t amoe_permute_workspace_bytes(int R, int E)
+{
+    if (R <= 0 || E <= 0) return 0;
+    return (size_t)permute_chunks(R) * (size_t)E * sizeof(int32_t);
+}
+
+AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, int T, int K, int E, int32_t* counts, int32_t* offsets,
+                                  int32_t* token_of, int32_t* slot_of, int32_t* row_of, void* workspace,
+                                  size_t workspace_bytes, void* stream)
+{
+    AMOE_REQUIRE(assign && counts && offsets && token_of && slot_of && row_of && workspace, AMOE_ERR_BAD_ARG,
+                 "permute_plan: null pointer");
+    AMOE_REQUIRE(T > 0 && K > 0 && E > 0, AMOE_ERR_BAD_ARG, "permute_plan: T, K, E must be positive");
+    AMOE_REQUIRE(E <= AMOE_MAX_EXPERTS, AMOE_ERR_UNSUPPORTED, "permute_plan: E=%d exceeds %d", E, AMOE_MAX_EXPERTS);
+    AMOE_REQUIRE((long long)T * K < (1ll << 31), AMOE_ERR_UNSUPPORTED, "permute_plan: T*K does not fit int32");
+    const int R = T * K;
+    AMOE_REQUIRE(workspace_bytes >= amoe_permute_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
+                 "permute_plan: workspace %zu < %zu bytes", workspace_bytes, amoe_permute_workspace_bytes(R, E));
+    const int n_chunks = permute_chunks(R);
+    const int n_blocks = (n_chunks + kWavesPerBlock - 1) / kWavesPerBlock;
+    hipStream_t s = (hipStream_t)stream;
+    int32_t* cc = (int32_t*)workspace;
+    hipLaunchKernelGGL(permute_hist_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E, R,
+                       n_chunks, cc);
+    hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(AMOE_MAX_EXPERTS), 0, s, cc, E, n_chunks, counts, offsets);
+    hipLaunchKernelGGL(permute_scatter_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E,
+                       R, n_chunks, cc, offsets, token_of, slot_of, row_of);
+    return amoe_check_launch("permute_plan");
+}

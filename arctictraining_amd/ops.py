@@ -1,0 +1,255 @@
+"""Thin tensor-level wrappers over the C ABI: allocate outputs with torch, pass raw device
+pointers and the current HIP stream, raise on error.  One function per stage of the
+expert layer, in the order the reference's forward runs them
+(arctic_training/model/moe/moe.py:219-323).
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+F32, BF16 = 0, 1
+ACT_SILU, ACT_GELU, ACT_RELU, ACT_GPT_OSS = 0, 1, 2, 3
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise RuntimeError(f"the expert-layer kernels support float32 and bfloat16, not {t.dtype}")
+
+
+def _chk(t: torch.Tensor, name: str, dtype=None) -> torch.Tensor:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (the HIP kernels have no CPU fallback)")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
+    return t
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def router_topk_fwd(logits: torch.Tensor, top_k: int, normalize: bool):
+    """logits [T,E] -> probs [T,E] f32, topk_idx [T,K] i32, scores [T,K] f32."""
+    lib = _lib.load()
+    _chk(logits, "logits")
+    T, E = logits.shape
+    probs = torch.empty((T, E), dtype=torch.float32, device=logits.device)
+    idx = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    scores = torch.empty((T, top_k), dtype=torch.float32, device=logits.device)
+    rc = lib.amoe_router_topk_fwd(
+        logits.data_ptr(), _dtype_code(logits), T, E, top_k, int(normalize), probs.data_ptr(), idx.data_ptr(),
+        scores.data_ptr(), _stream()
+    )
+    _lib.check(rc, "amoe_router_topk_fwd")
+    return probs, idx, scores
+
+
+def router_bwd(d_scores, probs, topk_idx, counts, out_dtype, normalize: bool, lb_coeff: float) -> torch.Tensor:
+    lib = _lib.load()
+    _chk(d_scores, "d_scores", torch.float32)
+    _chk(probs, "probs", torch.float32)
+    _chk(topk_idx, "topk_idx", torch.int32)
+    _chk(counts, "counts", torch.int32)
+    T, E = probs.shape
+    K = topk_idx.shape[1]
+    d_logits = torch.empty((T, E), dtype=out_dtype, device=probs.device)
+    rc = lib.amoe_router_bwd(
+        d_scores.data_ptr(), probs.data_ptr(), topk_idx.data_ptr(), counts.data_ptr(), _dtype_code(d_logits), T, E, K,
+        int(normalize), float(lb_coeff), d_logits.data_ptr(), _stream()
+    )
+    _lib.check(rc, "amoe_router_bwd")
+    return d_logits
+
+
+def permute_plan(assign: torch.Tensor, num_experts: int):
+    """assign [T,K] i32 -> counts [E], offsets [E+1], token_of [R], slot_of [R], row_of [T,K] (all i32)."""
+    lib = _lib.load()
+    _chk(assign, "assign", torch.int32)
+    T, K = assign.shape
+    R, E, dev = T * K, num_experts, assign.device
+    counts = torch.empty(E, dtype=torch.int32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    token_of = torch.empty(R, dtype=torch.int32, device=dev)
+    slot_of = torch.empty(R, dtype=torch.int32, device=dev)
+    row_of = torch.empty((T, K), dtype=torch.int32, device=dev)
+    ws_bytes = lib.amoe_permute_workspace_bytes(R, E)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    rc = lib.amoe_permute_plan(
+        assign.data_ptr(), T, K, E, counts.data_ptr(), offsets.data_ptr(), token_of.data_ptr(), slot_of.data_ptr(),
+        row_of.data_ptr(), ws.data_ptr(), ws.numel(), _stream()
+    )
+    _lib.check(rc, "amoe_permute_plan")
+    return counts, offsets, token_of, slot_of, row_of
+
+
+def gather_rows_fwd(x: torch.Tensor, token_of: torch.Tensor) -> torch.Tensor:
+    lib = _lib.load()
+    _chk(x, "x")
+    _chk(token_of, "token_of", torch.int32)
+    R, H = token_of.numel(), x.shape[1]
+    xp = torch.empty((R, H), dtype=x.dtype, device=x.device)
+    rc = lib.amoe_gather_rows_fwd(x.data_ptr(), token_of.data_ptr(), xp.data_ptr(), _dtype_code(x), R, H, _stream())
+    _lib.check(rc, "amoe_gather_rows_fwd")
+    return xp
+
+
+def gather_rows_bwd(d_xp: torch.Tensor, row_of: torch.Tensor, addend: Optional[torch.Tensor] = None) -> torch.Tensor:
+    lib = _lib.load()
+    _chk(d_xp, "d_xp")
+    _chk(row_of, "row_of", torch.int32)
+    if addend is not None:
+        _chk(addend, "addend", d_xp.dtype)
+    T, K = row_of.shape
+    H = d_xp.shape[1]
+    dx = torch.empty((T, H), dtype=d_xp.dtype, device=d_xp.device)
+    rc = lib.amoe_gather_rows_bwd(
+        d_xp.data_ptr(), row_of.data_ptr(), _ptr(addend), dx.data_ptr(), _dtype_code(d_xp), T, K, H, _stream()
+    )
+    _lib.check(rc, "amoe_gather_rows_bwd")
+    return dx
+
+
+def combine_fwd(moe_out: torch.Tensor, row_of: torch.Tensor, scores: torch.Tensor) -> torch.Tensor:
+    lib = _lib.load()
+    _chk(moe_out, "moe_out")
+    _chk(row_of, "row_of", torch.int32)
+    _chk(scores, "scores", torch.float32)
+    T, K = row_of.shape
+    H = moe_out.shape[1]
+    y = torch.empty((T, H), dtype=moe_out.dtype, device=moe_out.device)
+    rc = lib.amoe_combine_fwd(
+        moe_out.data_ptr(), row_of.data_ptr(), scores.data_ptr(), y.data_ptr(), _dtype_code(moe_out), T, K, H, _stream()
+    )
+    _lib.check(rc, "amoe_combine_fwd")
+    return y
+
+
+def combine_bwd(dy, moe_out, row_of, scores, need_d_out: bool = True) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+    lib = _lib.load()
+    _chk(dy, "dy", moe_out.dtype)
+    _chk(moe_out, "moe_out")
+    _chk(row_of, "row_of", torch.int32)
+    _chk(scores, "scores", torch.float32)
+    T, K = row_of.shape
+    H = moe_out.shape[1]
+    d_out = torch.empty_like(moe_out) if need_d_out else None
+    d_scores = torch.empty((T, K), dtype=torch.float32, device=dy.device)
+    rc = lib.amoe_combine_bwd(
+        dy.data_ptr(), moe_out.data_ptr(), row_of.data_ptr(), scores.data_ptr(), _ptr(d_out), d_scores.data_ptr(),
+        _dtype_code(dy), T, K, H, _stream()
+    )
+    _lib.check(rc, "amoe_combine_bwd")
+    return d_out, d_scores
+
+
+def _gemm_workspace(R: int, E: int, device) -> torch.Tensor:
+    n = _lib.load().amoe_grouped_gemm_workspace_bytes(R, E)
+    return torch.empty(max(n, 16), dtype=torch.uint8, device=device)
+
+
+def grouped_gemm_gateup_act_fwd(
+    xp: torch.Tensor,
+    w_gate_up: torch.Tensor,
+    offsets: torch.Tensor,
+    act: int = ACT_SILU,
+    a_row_map: Optional[torch.Tensor] = None,
+    n_rows: Optional[int] = None,
+    tile_cfg: int = 0,
+    want_gate_up: bool = True,
+):
+    """gate_up [R,2I], inter [R,I] from xp [R,H] (or x [T,H] with a_row_map [R]) and w [E,H,2I]."""
+    lib = _lib.load()
+    _chk(xp, "xp")
+    _chk(w_gate_up, "w_gate_up", xp.dtype)
+    _chk(offsets, "offsets", torch.int32)
+    if a_row_map is not None:
+        _chk(a_row_map, "a_row_map", torch.int32)
+    E, H, I2 = w_gate_up.shape
+    R = int(n_rows if n_rows is not None else (a_row_map.numel() if a_row_map is not None else xp.shape[0]))
+    I = I2 // 2
+    gate_up = torch.empty((R, I2), dtype=xp.dtype, device=xp.device) if want_gate_up else None
+    inter = torch.empty((R, I), dtype=xp.dtype, device=xp.device)
+    ws = _gemm_workspace(R, E, xp.device)
+    rc = lib.amoe_grouped_gemm_gateup_act_fwd(
+        xp.data_ptr(), _ptr(a_row_map), w_gate_up.data_ptr(), offsets.data_ptr(), _ptr(gate_up), inter.data_ptr(),
+        _dtype_code(xp), R, E, H, I, act, ws.data_ptr(), ws.numel(), tile_cfg, _stream()
+    )
+    _lib.check(rc, "amoe_grouped_gemm_gateup_act_fwd")
+    return gate_up, inter
+
+
+def grouped_gemm_nn(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 0) -> torch.Tensor:
+    """C[rows_e,:] = A[rows_e,:] @ B[e];  A [R,Kd], B [E,Kd,N] -> C [R,N]."""
+    lib = _lib.load()
+    _chk(A, "A")
+    _chk(B, "B", A.dtype)
+    _chk(offsets, "offsets", torch.int32)
+    E, Kd, N = B.shape
+    R = int(n_rows if n_rows is not None else (a_row_map.numel() if a_row_map is not None else A.shape[0]))
+    C = torch.empty((R, N), dtype=A.dtype, device=A.device)
+    ws = _gemm_workspace(R, E, A.device)
+    rc = lib.amoe_grouped_gemm_nn(
+        A.data_ptr(), _ptr(a_row_map), B.data_ptr(), offsets.data_ptr(), C.data_ptr(), _dtype_code(A), R, E, Kd, N,
+        ws.data_ptr(), ws.numel(), tile_cfg, _stream()
+    )
+    _lib.check(rc, "amoe_grouped_gemm_nn")
+    return C
+
+
+def grouped_gemm_nt(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 0) -> torch.Tensor:
+    """C[rows_e,:] = A[rows_e,:] @ B[e]^T;  A [R,N], B [E,Kd,N] -> C [R,Kd]."""
+    lib = _lib.load()
+    _chk(A, "A")
+    _chk(B, "B", A.dtype)
+    _chk(offsets, "offsets", torch.int32)
+    E, Kd, N = B.shape
+    R = int(n_rows if n_rows is not None else (a_row_map.numel() if a_row_map is not None else A.shape[0]))
+    C = torch.empty((R, Kd), dtype=A.dtype, device=A.device)
+    ws = _gemm_workspace(R, E, A.device)
+    rc = lib.amoe_grouped_gemm_nt(
+        A.data_ptr(), _ptr(a_row_map), B.data_ptr(), offsets.data_ptr(), C.data_ptr(), _dtype_code(A), R, E, Kd, N,
+        ws.data_ptr(), ws.numel(), tile_cfg, _stream()
+    )
+    _lib.check(rc, "amoe_grouped_gemm_nt")
+    return C
+
+
+def grouped_gemm_wgrad(A, B, offsets, num_experts: int, tile_cfg: int = 0) -> torch.Tensor:
+    """C[e] = A[rows_e,:]^T @ B[rows_e,:];  A [R,Kd], B [R,N] -> C [E,Kd,N]."""
+    lib = _lib.load()
+    _chk(A, "A")
+    _chk(B, "B", A.dtype)
+    _chk(offsets, "offsets", torch.int32)
+    R, Kd = A.shape
+    N = B.shape[1]
+    C = torch.empty((num_experts, Kd, N), dtype=A.dtype, device=A.device)
+    rc = lib.amoe_grouped_gemm_wgrad(
+        A.data_ptr(), B.data_ptr(), offsets.data_ptr(), C.data_ptr(), _dtype_code(A), R, num_experts, Kd, N, tile_cfg,
+        _stream()
+    )
+    _lib.check(rc, "amoe_grouped_gemm_wgrad")
+    return C
+
+
+def gated_act_bwd(gate_up: torch.Tensor, d_inter: torch.Tensor, act: int = ACT_SILU) -> torch.Tensor:
+    lib = _lib.load()
+    _chk(gate_up, "gate_up")
+    _chk(d_inter, "d_inter", gate_up.dtype)
+    R, I = d_inter.shape
+    d_gu = torch.empty_like(gate_up)
+    rc = lib.amoe_gated_act_bwd(
+        gate_up.data_ptr(), d_inter.data_ptr(), d_gu.data_ptr(), _dtype_code(gate_up), R, I, act, _stream()
+    )
+    _lib.check(rc, "amoe_gated_act_bwd")
+    return d_gu

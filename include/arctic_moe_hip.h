@@ -1,0 +1,171 @@
+/*
+ * C ABI of libarctic_moe_hip.so -- the MI355X (gfx950) expert-layer kernels that stand where
+ * the reference binds its pybind11 module `ragged_ops`
+ * (arctic_training/kernels/moe_ops/ragged_ops.cpp:12-26) and where its default path calls
+ * torch ops (arctic_training/model/moe/moe.py:54-60, 176-193, 340-411, 450-461).
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes only; every pointer is DEVICE memory owned by the caller
+ *     (the reference's functions likewise fill caller-allocated tensors in place,
+ *     top_k_gating.h:15-35, moe_scatter.h:16-29);
+ *   - the library never allocates, frees or keeps a pointer past return;
+ *   - `stream` is a hipStream_t passed as void*; work is stream-ordered, no host sync;
+ *   - return 0 on success or a negative AMOE_ERR_* code; arguments are validated before
+ *     the first HIP call, so argument errors can be exercised without a GPU;
+ *     amoe_last_error() returns the calling thread's last message;
+ *   - dtype: AMOE_F32 or AMOE_BF16 for activations / weights; probabilities, scores and
+ *     score gradients are always float32; indices are int32 (routed rows R = T*K < 2^31);
+ *   - routed-row order is the reference's (moe.py:367-382): grouped by expert ascending,
+ *     inside an expert ascending flat slot f = k*T + t.
+ */
+#ifndef ARCTIC_MOE_HIP_H
+#define ARCTIC_MOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AMOE_OK 0
+#define AMOE_ERR_BAD_ARG (-1)     /* null pointer, non-positive size, bad enum */
+#define AMOE_ERR_UNSUPPORTED (-2) /* shape outside what the kernels cover */
+#define AMOE_ERR_WORKSPACE (-3)   /* workspace too small */
+#define AMOE_ERR_LAUNCH (-4)      /* HIP reported a launch failure */
+
+#define AMOE_F32 0
+#define AMOE_BF16 1
+
+#define AMOE_ACT_SILU 0
+#define AMOE_ACT_GELU 1
+#define AMOE_ACT_RELU 2
+#define AMOE_ACT_GPT_OSS 3 /* x * sigmoid(1.702 x), utils.py:118-123 */
+
+#define AMOE_MAX_EXPERTS 512
+#define AMOE_MAX_TOPK 16
+
+/* library version (major*10000 + minor*100 + patch) */
+int amoe_version(void);
+/* message of the last error on the calling thread ("" if none) */
+const char* amoe_last_error(void);
+
+/*
+ * Router softmax + top-k.  Replaces top_k_gating (top_k_gating.h:15-22,
+ * top_k_gating_cuda.cu:74-147) and moe.py:360-366.
+ *   logits [T,E] dtype  ->  probs [T,E] f32 (softmax evaluated in f32),
+ *   topk_idx [T,K] i32 (value descending, lowest expert index first among equal logits),
+ *   scores [T,K] f32 = the selected probabilities, divided by their sum when `normalize`,
+ *   then rounded through `dtype` (the reference casts the scores to the model dtype).
+ */
+int amoe_router_topk_fwd(const void* logits, int dtype, int T, int E, int K, int normalize, float* probs,
+                         int32_t* topk_idx, float* scores, void* stream);
+
+/*
+ * Router backward.  Replaces top_k_gating_bwd (top_k_gating.h:24-28,
+ * top_k_gating_cuda.cu:243-294) plus the load-balance hook moe.py:393-406.
+ *   d_scores [T,K] f32, probs [T,E] f32, topk_idx [T,K], counts [E] i32 (routed rows per
+ *   expert) -> d_logits [T,E] dtype.
+ *   d_probs = scatter(normalise-backward(d_scores)) + lb_coeff * counts/sum(counts);
+ *   d_logits = probs * (d_probs - sum_e probs*d_probs).   lb_coeff = loss_coeff / T / ep_size.
+ */
+int amoe_router_bwd(const float* d_scores, const float* probs, const int32_t* topk_idx, const int32_t* counts,
+                    int dtype, int T, int E, int K, int normalize, float lb_coeff, void* d_logits, void* stream);
+
+/*
+ * Permutation plan.  Replaces the atomics of top_k_gating plus the prefix sum and slot
+ * computation of moe_scatter (moe_scatter_cuda.cu:69-139) with the deterministic order of
+ * moe.py:367-382.
+ *   assign [T,K] i32 (expert of slot (t,k)) ->
+ *   counts [E], offsets [E+1] (exclusive prefix), token_of [R] (row -> token, the
+ *   reference's token_mapped_slots), slot_of [R] (row -> flat slot f = k*T+t, the
+ *   reference's pre-modulo permutation), row_of [T,K] (slot -> row, the custom path's
+ *   mapped_slots).  workspace: amoe_permute_workspace_bytes(T*K, E) bytes.
+ */
+size_t amoe_permute_workspace_bytes(int R, int E);
+int amoe_permute_plan(const int32_t* assign, int T, int K, int E, int32_t* counts, int32_t* offsets,
+                      int32_t* token_of, int32_t* slot_of, int32_t* row_of, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+/*
+ * Row gather  xp[r,:] = x[token_of[r],:]  (moe.py:356; forward half of moe_scatter,
+ * moe_scatter_cuda.cu:141-154).  x [T,H], xp [R,H].
+ */
+int amoe_gather_rows_fwd(const void* x, const int32_t* token_of, void* xp, int dtype, int R, int H, void* stream);
+
+/*
+ * Backward of the row gather (moe_scatter_backward, moe_scatter.h:25-29):
+ *   dx[t,:] = (addend ? addend[t,:] : 0) + sum_k d_xp[row_of[t,k],:]   (f32 accumulate)
+ */
+int amoe_gather_rows_bwd(const void* d_xp, const int32_t* row_of, const void* addend, void* dx, int dtype, int T,
+                         int K, int H, void* stream);
+
+/*
+ * Weighted combine  y[t,:] = sum_k scores[t,k] * moe_out[row_of[t,k],:]  (moe.py:450-461;
+ * moe_gather, moe_gather.cpp:28-60), f32 accumulate, one rounding.
+ */
+int amoe_combine_fwd(const void* moe_out, const int32_t* row_of, const float* scores, void* y, int dtype, int T,
+                     int K, int H, void* stream);
+
+/*
+ * Backward of the combine (moe_gather_backward, moe_gather.cpp:75-102) as the true
+ * derivative of the forward above:
+ *   d_moe_out[row_of[t,k],:] = dy[t,:] * scores[t,k];   d_scores[t,k] = <dy[t,:], moe_out[row,:]>.
+ * d_moe_out may be null (only d_scores wanted).
+ */
+int amoe_combine_bwd(const void* dy, const void* moe_out, const int32_t* row_of, const float* scores,
+                     void* d_moe_out, float* d_scores, int dtype, int T, int K, int H, void* stream);
+
+/* workspace every grouped GEMM below needs (tile map built on the device from offsets) */
+size_t amoe_grouped_gemm_workspace_bytes(int R, int E);
+
+/*
+ * Grouped gate_up GEMM with the gated activation fused (moe.py:54-60 + 187-191):
+ *   gate_up[rows_e, :] = xp[rows_e, :] @ w_gate_up[e]          [R,2I]
+ *   inter[r, i] = gate_up[r, 2i+1] * act(gate_up[r, 2i])        [R,I]
+ * xp [R,H]; w_gate_up [E,H,2I] (gate in even, up in odd columns); offsets [E+1].
+ * When `a_row_map` is non-null, row r of the A operand is read from xp[a_row_map[r], :]
+ * (the gather of moe.py:356 folded into the GEMM; xp is then the un-permuted [T,H]).
+ * gate_up may be null when only inter is wanted.  tile_cfg: 0 = library default.
+ */
+int amoe_grouped_gemm_gateup_act_fwd(const void* xp, const int32_t* a_row_map, const void* w_gate_up,
+                                     const int32_t* offsets, void* gate_up, void* inter, int dtype, int R, int E,
+                                     int H, int I, int act, void* workspace, size_t workspace_bytes, int tile_cfg,
+                                     void* stream);
+
+/*
+ * Grouped GEMM, B not transposed (moe.py:54-60):  C[rows_e,:] = A[rows_e,:] @ B[e]
+ * A [R,Kd] (rows optionally gathered through a_row_map), B [E,Kd,N], C [R,N].  Used for
+ * the down projection.
+ */
+int amoe_grouped_gemm_nn(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C,
+                         int dtype, int R, int E, int Kd, int N, void* workspace, size_t workspace_bytes,
+                         int tile_cfg, void* stream);
+
+/*
+ * Grouped data-gradient GEMM:  C[rows_e,:] = A[rows_e,:] @ B[e]^T
+ * A [R,N], B [E,Kd,N] (the forward weight), C [R,Kd].  The autograd of moe.py:59 w.r.t. A.
+ */
+int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C,
+                         int dtype, int R, int E, int Kd, int N, void* workspace, size_t workspace_bytes,
+                         int tile_cfg, void* stream);
+
+/*
+ * Grouped weight-gradient GEMM:  C[e] = A[rows_e,:]^T @ B[rows_e,:]   (zeros for an empty
+ * expert).  A [R,Kd], B [R,N], C [E,Kd,N].  The autograd of moe.py:59 w.r.t. B[e].
+ */
+int amoe_grouped_gemm_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int dtype, int R, int E,
+                            int Kd, int N, int tile_cfg, void* stream);
+
+/*
+ * Backward of the gated activation (autograd of moe.py:189-191):
+ *   d_gate_up[r,2i]   = d_inter[r,i] * up * act'(gate)
+ *   d_gate_up[r,2i+1] = d_inter[r,i] * act(gate)
+ */
+int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, void* d_gate_up, int dtype, int R, int I, int act,
+                       void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARCTIC_MOE_HIP_H */

@@ -1,0 +1,210 @@
+"""Whole-layer parity: the ArcticMoE module (HIP kernels through the C ABI, forward and
+backward) against the CPU oracle on the same seeded inputs.
+
+Routing (top-k indices, per-expert counts, permutation order) must be bit-exact given the
+logits the layer itself computed; outputs and gradients must agree with the oracle
+evaluated in float64 from the same rounded inputs to rel-L2 <= 1e-2 (bf16) / 1e-5 (float32).
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# name: (dtype, T, H, E, K, I, extra make_inputs kwargs)  -- the BASELINE configurations,
+# the first at full size, the bf16 ones scaled down so the float64 oracle runs in seconds
+CONFIGS = {
+    "c1_full_fp32": (torch.float32, 2048, 512, 8, 2, 1024, {}),
+    "c2_mixtral_scaled": (torch.bfloat16, 1024, 512, 8, 2, 1792, {}),
+    "c3_qwen3_scaled": (torch.bfloat16, 2048, 256, 128, 8, 192, {}),
+    "c5_stress_scaled": (torch.bfloat16, 4096, 256, 64, 4, 192, dict(bias_hot=0.55, n_hot=4, n_dead=8)),
+    "tiny_fp32": (torch.float32, 37, 64, 5, 3, 32, {}),
+    "tiny_bf16_k1": (torch.bfloat16, 130, 64, 4, 1, 64, {}),
+}
+
+
+def build_layer(dtype, H, E, K, I, device, normalize=True, loss_coeff=0.001, act=F.silu, **kw):
+    from arctictraining_amd import ArcticMoE, MoEConfig
+
+    cfg = MoEConfig(
+        act_fn=act,
+        input_dtype=dtype,
+        intermediate_dim=I,
+        model_dim=H,
+        normalize_topk_scores=normalize,
+        num_experts=E,
+        top_k=K,
+        loss_coeff=loss_coeff,
+        **kw,
+    )
+    return ArcticMoE(cfg).to(device)
+
+
+def run_layer(layer, x, wr, wgu, wd, dy, device, replay=None):
+    with torch.no_grad():
+        layer.router_gate.copy_(wr)
+        layer.expert_gate_up.copy_(wgu)
+        layer.expert_down.copy_(wd)
+    for p in layer.parameters():
+        p.grad = None
+    layer.capture = {}
+    xg = x.to(device).requires_grad_(True)
+    out = layer(xg, replay) if replay is not None else layer(xg)
+    y = out[0] if isinstance(out, tuple) else out
+    y.backward(dy.to(device))
+    torch.cuda.synchronize()
+    return dict(
+        y=y.detach().cpu(),
+        dx=xg.grad.cpu(),
+        d_router_gate=layer.router_gate.grad.cpu(),
+        d_expert_gate_up=layer.expert_gate_up.grad.cpu(),
+        d_expert_down=layer.expert_down.grad.cpu(),
+        cap={k: v.cpu() for k, v in layer.capture.items()},
+        out=out,
+    )
+
+
+def check_against_oracle(got, x, wr, wgu, wd, dy, ocfg, dtype, replay=None):
+    cap = got["cap"]
+    ref = O.forward_backward(
+        x, wr, wgu, wd, dy, ocfg, compute_dtype=torch.float64, logits_for_selection=cap["logits"],
+        replay_assignments=replay,
+    )
+    T, K = cap["topk_idx"].shape
+    # ---- bit-exact routing
+    assert torch.equal(cap["topk_idx"].long(), ref["topk_idx"]), "top-k indices"
+    assert torch.equal(cap["counts"].long(), ref["counts"]), "per-expert counts"
+    assert torch.equal(cap["slot_of"].long(), ref["perm"]), "permutation order"
+    assert torch.equal(cap["token_of"].long(), ref["token_ids"]), "token ids"
+    assert torch.equal(cap["row_of"].long(), O.inverse_row_map(ref["perm"], T, K)), "inverse map"
+    # the layer's logits are the oracle's up to the rounding of the model dtype
+    assert O.rel_l2(cap["logits"], ref["logits"]) <= (1e-2 if dtype == torch.bfloat16 else 1e-5)
+    # ---- values
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-5
+    errs = {k: O.rel_l2(got[k], ref[k]) for k in ("y", "dx", "d_router_gate", "d_expert_gate_up", "d_expert_down")}
+    print("rel-L2:", {k: f"{v:.2e}" for k, v in errs.items()}, flush=True)
+    for k, v in errs.items():
+        assert v <= tol, f"{k}: rel-L2 {v:.3e} > {tol}"
+    return ref, errs
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_layer_matches_oracle(gpu_device, name):
+    dtype, T, H, E, K, I, extra = CONFIGS[name]
+    print("layer", name, flush=True)
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=1234, **extra)
+    layer = build_layer(dtype, H, E, K, I, gpu_device)
+    got = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001)
+    ref, _ = check_against_oracle(got, x, wr, wgu, wd, dy, ocfg, dtype)
+    if name == "c5_stress_scaled":
+        counts = ref["counts"]
+        assert int((counts[-8:] == 0).sum()) == 8, "the biased router must starve the last 8 experts"
+        assert 0.35 < float(counts[:4].sum()) / float(counts.sum()) < 0.65
+        assert bool((got["d_expert_gate_up"][-8:] == 0).all()) and bool((got["d_expert_down"][-8:] == 0).all())
+
+
+def test_layer_3d_input_and_no_normalisation(gpu_device):
+    dtype, T, H, E, K, I = torch.bfloat16, 512, 128, 16, 4, 64
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=5)
+    layer = build_layer(dtype, H, E, K, I, gpu_device, normalize=False, loss_coeff=0.05)
+    got = run_layer(layer, x.view(4, T // 4, H), wr, wgu, wd, dy.view(4, T // 4, H), gpu_device)
+    assert got["y"].shape == (4, T // 4, H)
+    ocfg = O.OracleConfig(
+        model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.05, normalize_topk_scores=False
+    )
+    got["y"], got["dx"] = got["y"].view(T, H), got["dx"].view(T, H)
+    check_against_oracle(got, x, wr, wgu, wd, dy, ocfg, dtype)
+
+
+def test_layer_load_balance_term(gpu_device):
+    """The load-balance gradient (moe.py:393-406) changes d_router_gate and dx only, by
+    the amount the oracle predicts."""
+    dtype, T, H, E, K, I = torch.float32, 256, 64, 8, 2, 64
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=6)
+    res = {}
+    for coeff in (0.0, 5.0):
+        layer = build_layer(dtype, H, E, K, I, gpu_device, loss_coeff=coeff)
+        res[coeff] = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+        ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=coeff)
+        check_against_oracle(res[coeff], x, wr, wgu, wd, dy, ocfg, dtype)
+    assert torch.equal(res[0.0]["d_expert_down"], res[5.0]["d_expert_down"])
+    assert not torch.equal(res[0.0]["d_router_gate"], res[5.0]["d_router_gate"])
+
+
+def test_layer_routing_replay_and_returned_scores(gpu_device):
+    """With replay the rows go to the replayed experts while the scores stay those of the
+    layer's own top-k (moe.py:363-372); return_router_scores returns them in row order."""
+    dtype, T, H, E, K, I = torch.bfloat16, 300, 128, 8, 2, 64
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=8)
+    g = torch.Generator().manual_seed(9)
+    replay = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    layer = build_layer(
+        dtype, H, E, K, I, gpu_device, enable_routing_replay=True, return_router_scores=True
+    )
+    got = run_layer(layer, x, wr, wgu, wd, dy, gpu_device, replay=replay.to(gpu_device))
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001)
+    ref, _ = check_against_oracle(got, x, wr, wgu, wd, dy, ocfg, dtype, replay=replay)
+    y, scores = got["out"]
+    assert scores.shape == (T * K,) and scores.dtype == dtype
+    assert O.rel_l2(scores.cpu(), ref["scores_perm"]) <= 1e-2
+    with pytest.raises(AssertionError):
+        layer(x.to(gpu_device))
+
+
+def test_layer_shared_expert(gpu_device):
+    """Shared expert with a sigmoid output gate (moe.py:305-314) on top of the routed path."""
+    dtype, T, H, E, K, I = torch.float32, 128, 64, 4, 2, 32
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=10)
+    layer = build_layer(dtype, H, E, K, I, gpu_device, use_shared_expert=True)
+    g = torch.Generator().manual_seed(11)
+    sgu, sd, sg = (torch.randn(s, generator=g) * 0.05 for s in ((H, 2 * I), (I, H), (H, 1)))
+    with torch.no_grad():
+        layer.shared_expert_gate_up.copy_(sgu)
+        layer.shared_expert_down.copy_(sd)
+        layer.shared_expert_output_gate.copy_(sg)
+    got = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001)
+    ref = O.forward(x, wr, wgu, wd, ocfg, compute_dtype=torch.float64, logits_for_selection=got["cap"]["logits"])
+    x64 = x.double()
+    s_i = x64 @ sgu.double()
+    s_out = (s_i[:, 1::2] * F.silu(s_i[:, 0::2])) @ sd.double()
+    expect = ref["y"] + s_out * torch.sigmoid(x64 @ sg.double())
+    assert O.rel_l2(got["y"], expect) <= 1e-5
+    assert layer.shared_expert_down.grad is not None
+
+
+def test_layer_is_deterministic(gpu_device):
+    dtype, T, H, E, K, I = torch.bfloat16, 1024, 256, 32, 4, 128
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=13)
+    layer = build_layer(dtype, H, E, K, I, gpu_device)
+    a = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+    b = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+    for k in ("y", "dx", "d_router_gate", "d_expert_gate_up", "d_expert_down"):
+        assert torch.equal(a[k], b[k]), f"{k} differs between two identical runs"
+
+
+def test_module_surface(gpu_device):
+    """Names, shapes and attributes the reference's callers rely on (moe.py:91-130,
+    utils.py:61-68, 350-369, 449-461)."""
+    layer = build_layer(torch.bfloat16, 128, 8, 2, 64, gpu_device, use_shared_expert=True)
+    names = dict(layer.named_parameters())
+    assert set(names) == {
+        "router_gate", "expert_gate_up", "expert_down", "shared_expert_gate_up", "shared_expert_down",
+        "shared_expert_output_gate",
+    }
+    assert names["router_gate"].shape == (8, 128)
+    assert names["expert_gate_up"].shape == (8, 128, 128)
+    assert names["expert_down"].shape == (8, 64, 128)
+    assert layer.num_local_experts == 8 and layer.ep_size == 1 and layer.ep_rank == 0
+    assert layer._config.use_shared_expert
+    layer.enable_wall_clock_breakdown()
+    assert layer.timers.wall_clock_breakdown
+    x = torch.randn(16, 128, device=gpu_device, dtype=torch.bfloat16)
+    for p in layer.parameters():
+        torch.nn.init.normal_(p, std=0.02)
+    layer(x)
+    assert layer.timers.elapsed("amoe e2e") > 0 and layer.timers.elapsed("groupGeMM") > 0
+    assert "expert_gate_up" in repr(layer)

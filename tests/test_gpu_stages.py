@@ -1,0 +1,342 @@
+"""Stage-level parity of the HIP kernels (through the C ABI) against the CPU oracle.
+
+Integer results (top-k indices, counts, offsets, the three index maps) must be bit-exact;
+floating-point results are compared by relative L2 error against the oracle evaluated in
+float64 from the same (already rounded) inputs: <= 1e-2 for bf16 data, <= 1e-5 for float32.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 1e-2
+F32_TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def ops(gpu_device):
+    from arctictraining_amd import ops as _ops
+
+    return _ops
+
+
+def _tol(dtype):
+    return BF16_TOL if dtype == torch.bfloat16 else F32_TOL
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------------ router
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("E,K", [(8, 2), (64, 4), (128, 8), (60, 6), (256, 8), (384, 1), (512, 16), (5, 5)])
+@pytest.mark.parametrize("normalize", [True, False])
+def test_router_topk(ops, gpu_device, dtype, E, K, normalize):
+    _say("router_topk", dtype, E, K, normalize)
+    g = torch.Generator().manual_seed(E * 131 + K)
+    T = 777
+    logits = (torch.randn(T, E, generator=g) * 0.9).to(dtype)
+    # rows with forced ties, including across the k / k+1 boundary and an all-equal row
+    logits[0] = 0.0
+    logits[1, : E // 2] = 1.5
+    logits[2, :5] = torch.tensor([0.25, -0.0, 0.0, 0.25, 0.5]).to(dtype)
+    probs, idx, scores = ops.router_topk_fwd(logits.to(gpu_device), K, normalize)
+    torch.cuda.synchronize()
+    ref_p = O.softmax_probs(logits)
+    _, ref_idx = O.topk_canonical(logits.to(torch.float64) + 0.0, K)
+    assert torch.equal(idx.cpu().to(torch.int64), ref_idx), "top-k indices must be bit-exact"
+    assert torch.allclose(probs.cpu(), ref_p, atol=2e-7, rtol=2e-6)
+    ref_s = O.normalize_and_cast(torch.gather(ref_p, -1, ref_idx), normalize, dtype).float()
+    got_s = scores.cpu()
+    # the scores went through the model dtype: allow one unit in the last place of it
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -21
+    assert torch.all((got_s - ref_s).abs() <= ulp * ref_s.abs() + 1e-9)
+    if dtype == torch.bfloat16:
+        assert torch.equal(got_s, got_s.to(torch.bfloat16).float()), "scores are bf16-representable"
+
+
+def test_router_topk_matches_selection_on_probabilities(ops, gpu_device):
+    """On configuration-shaped logits the selection on logits equals the reference's
+    selection on float32 probabilities (with the lowest-index tie rule)."""
+    x, wr, *_ = O.make_inputs(4096, 256, 128, 8, 8, torch.bfloat16, seed=12)
+    logits = O.router_linear(x, wr)
+    assert O.selection_agrees(logits, 8)
+    _, idx, _ = ops.router_topk_fwd(logits.to(gpu_device), 8, True)
+    _, ref = O.topk_canonical(O.softmax_probs(logits), 8)
+    assert torch.equal(idx.cpu().long(), ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("E,K,normalize", [(8, 2, True), (128, 8, True), (64, 4, False), (300, 3, True)])
+def test_router_bwd(ops, gpu_device, dtype, E, K, normalize):
+    _say("router_bwd", dtype, E, K, normalize)
+    g = torch.Generator().manual_seed(E + K)
+    T = 333
+    logits = (torch.randn(T, E, generator=g)).to(dtype)
+    probs = O.softmax_probs(logits)
+    _, idx = O.topk_canonical(logits.double(), K)
+    d_scores = torch.randn(T, K, generator=g)
+    counts = torch.randint(0, 50, (E,), generator=g, dtype=torch.int32)
+    lb = 0.37 / T
+    got = ops.router_bwd(
+        d_scores.to(gpu_device), probs.to(gpu_device), idx.to(torch.int32).to(gpu_device), counts.to(gpu_device), dtype,
+        normalize, lb,
+    )
+    p = probs.double()
+    pt = torch.gather(p, -1, idx)
+    ds = d_scores.double()
+    if normalize:
+        S = pt.sum(-1, keepdim=True)
+        dpt = (ds - (ds * pt / S).sum(-1, keepdim=True)) / S
+    else:
+        dpt = ds
+    dp = torch.zeros_like(p).scatter_add(-1, idx, dpt) + lb * counts.double()[None] / counts.sum()
+    ref = p * (dp - (p * dp).sum(-1, keepdim=True))
+    assert O.rel_l2(got.cpu(), ref) <= (4e-3 if dtype == torch.bfloat16 else F32_TOL)
+
+
+# ------------------------------------------------------------------ permutation
+def _check_plan(ops, dev, assign, E):
+    T, K = assign.shape
+    counts, offsets, token_of, slot_of, row_of = ops.permute_plan(assign.to(torch.int32).to(dev), E)
+    torch.cuda.synchronize()
+    perm, tok, cnt = O.permutation(assign.long(), E)
+    assert torch.equal(counts.cpu().long(), cnt), "counts"
+    assert torch.equal(offsets.cpu().long(), torch.cat([torch.zeros(1, dtype=torch.int64), cnt.cumsum(0)])), "offsets"
+    assert torch.equal(slot_of.cpu().long(), perm), "permutation order"
+    assert torch.equal(token_of.cpu().long(), tok), "token ids"
+    assert torch.equal(row_of.cpu().long(), O.inverse_row_map(perm, T, K)), "inverse map"
+
+
+@pytest.mark.parametrize(
+    "T,K,E",
+    [(3, 2, 2), (1, 1, 1), (64, 1, 8), (1000, 2, 8), (1025, 4, 64), (4096, 8, 128), (777, 3, 300), (5000, 6, 512)],
+)
+def test_permute_plan_random(ops, gpu_device, T, K, E):
+    _say("permute_plan", T, K, E)
+    g = torch.Generator().manual_seed(T + K + E)
+    assign = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    _check_plan(ops, gpu_device, assign, E)
+
+
+def test_permute_plan_worked_example(ops, gpu_device):
+    assign = torch.tensor([[1, 0], [0, 1], [1, 0]])
+    counts, offsets, token_of, slot_of, row_of = ops.permute_plan(assign.to(torch.int32).to(gpu_device), 2)
+    assert slot_of.tolist() == [1, 3, 5, 0, 2, 4]
+    assert token_of.tolist() == [1, 0, 2, 0, 2, 1]
+    assert counts.tolist() == [3, 3] and offsets.tolist() == [0, 3, 6]
+
+
+def test_permute_plan_skewed_and_empty(ops, gpu_device):
+    g = torch.Generator().manual_seed(3)
+    T, K, E = 6000, 4, 64
+    # 4 hot experts take about half, the last 8 experts receive nothing
+    w = torch.ones(E)
+    w[:4] = 13.0
+    w[-8:] = 0.0
+    assign = torch.multinomial(w.expand(T, E), K, replacement=False, generator=g)
+    _check_plan(ops, gpu_device, assign, E)
+    # everything to one expert per k
+    assign = torch.tensor([[5, 9]]).expand(3000, 2).contiguous()
+    _check_plan(ops, gpu_device, assign, 16)
+
+
+def test_permute_plan_full_size_headline(ops, gpu_device):
+    """T=16384, K=8, E=128 (the headline shape): bit-exact against the oracle."""
+    g = torch.Generator().manual_seed(7)
+    T, K, E = 16384, 8, 128
+    assign = torch.multinomial(torch.ones(T, E), K, replacement=False, generator=g)
+    _check_plan(ops, gpu_device, assign, E)
+
+
+# ------------------------------------------------------------------ row kernels
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,K,H,E", [(50, 2, 64, 4), (300, 8, 2048, 16), (129, 4, 520, 8)])
+def test_gather_and_combine(ops, gpu_device, dtype, T, K, H, E):
+    _say("rows", dtype, T, K, H, E)
+    g = torch.Generator().manual_seed(T + H)
+    assign = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    perm, tok, _ = O.permutation(assign, E)
+    row_of = O.inverse_row_map(perm, T, K)
+    R = T * K
+    x = torch.randn(T, H, generator=g).to(dtype)
+    d = gpu_device
+    tok_d, row_d = tok.to(torch.int32).to(d), row_of.to(torch.int32).to(d)
+
+    xp = ops.gather_rows_fwd(x.to(d), tok_d)
+    assert torch.equal(xp.cpu(), x[tok]), "gather is a copy: bit-exact"
+
+    d_xp = torch.randn(R, H, generator=g).to(dtype)
+    addend = torch.randn(T, H, generator=g).to(dtype)
+    dx = ops.gather_rows_bwd(d_xp.to(d), row_d, addend.to(d))
+    ref = addend.double().index_add(0, tok, d_xp.double())
+    assert O.rel_l2(dx.cpu(), ref) <= _tol(dtype)
+    dx = ops.gather_rows_bwd(d_xp.to(d), row_d, None)
+    ref = torch.zeros(T, H, dtype=torch.float64).index_add(0, tok, d_xp.double())
+    assert O.rel_l2(dx.cpu(), ref) <= _tol(dtype)
+
+    out = torch.randn(R, H, generator=g).to(dtype)
+    s_tk = torch.rand(T, K, generator=g).to(dtype).float()
+    s_perm = s_tk.t().reshape(-1)[perm]
+    y = ops.combine_fwd(out.to(d), row_d, s_tk.to(d))
+    ref = O.combine(out.double(), tok, s_perm.double(), K)
+    assert O.rel_l2(y.cpu(), ref) <= _tol(dtype)
+
+    dy = torch.randn(T, H, generator=g).to(dtype)
+    d_out, d_s = ops.combine_bwd(dy.to(d), out.to(d), row_d, s_tk.to(d))
+    ref_d_out = dy.double()[tok] * s_perm.double()[:, None]
+    ref_ds_perm = (dy.double()[tok] * out.double()).sum(-1)
+    ref_ds = torch.zeros(R, dtype=torch.float64)
+    ref_ds[perm] = ref_ds_perm
+    assert O.rel_l2(d_out.cpu(), ref_d_out) <= _tol(dtype)
+    assert O.rel_l2(d_s.cpu(), ref_ds.view(K, T).t()) <= 1e-5
+    _, d_s2 = ops.combine_bwd(dy.to(d), out.to(d), row_d, s_tk.to(d), need_d_out=False)
+    assert torch.equal(d_s2, d_s)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("act", ["silu", "gelu", "relu", "gpt_oss"])
+def test_gated_act_bwd(ops, gpu_device, dtype, act):
+    code = {"silu": 0, "gelu": 1, "relu": 2, "gpt_oss": 3}[act]
+    g = torch.Generator().manual_seed(4)
+    R, I = 100, 96
+    gu = torch.randn(R, 2 * I, generator=g).to(dtype)
+    di = torch.randn(R, I, generator=g).to(dtype)
+    got = ops.gated_act_bwd(gu.to(gpu_device), di.to(gpu_device), code)
+    gu64 = gu.double().requires_grad_(True)
+    inter = gu64[:, 1::2] * O.activation(act)(gu64[:, 0::2])
+    inter.backward(di.double())
+    assert O.rel_l2(got.cpu(), gu64.grad) <= (5e-3 if dtype == torch.bfloat16 else 2e-5)
+
+
+# ------------------------------------------------------------------ grouped GEMMs
+def _ragged_counts(name, R, E, g):
+    if name == "uniform":
+        c = torch.full((E,), R // E)
+        c[0] += R - int(c.sum())
+    elif name == "ragged":
+        w = torch.rand(E, generator=g) + 0.05
+        c = torch.floor(w / w.sum() * R).long()
+        c[-1] += R - int(c.sum())
+    elif name == "holes":  # empty experts, one-row experts, one dominant expert
+        c = torch.zeros(E, dtype=torch.long)
+        c[1] = 1
+        c[E // 2] = 3
+        c[E - 2] = R - 4
+    else:
+        raise ValueError(name)
+    assert int(c.sum()) == R and bool((c >= 0).all())
+    return c
+
+
+def _offsets(counts, dev):
+    return torch.cat([torch.zeros(1, dtype=torch.int64), counts.cumsum(0)]).to(torch.int32).to(dev)
+
+
+GEMM_CASES = [
+    # dtype, R, E, Kd, N, counts, tile_cfg
+    (torch.bfloat16, 512, 4, 64, 64, "uniform", 0),
+    (torch.bfloat16, 1000, 8, 128, 192, "ragged", 1),
+    (torch.bfloat16, 1000, 8, 128, 192, "ragged", 2),
+    (torch.bfloat16, 1000, 8, 128, 192, "ragged", 3),
+    (torch.bfloat16, 777, 6, 256, 320, "holes", 0),
+    (torch.bfloat16, 2500, 16, 512, 384, "ragged", 0),
+    (torch.bfloat16, 300, 3, 192, 1096, "ragged", 0),
+    (torch.float32, 512, 4, 64, 64, "uniform", 0),
+    (torch.float32, 777, 6, 100, 76, "holes", 0),
+    (torch.float32, 1000, 8, 128, 192, "ragged", 0),
+]
+
+
+@pytest.mark.parametrize("dtype,R,E,Kd,N,cname,cfg", GEMM_CASES)
+def test_grouped_gemm_nn_nt_wgrad(ops, gpu_device, dtype, R, E, Kd, N, cname, cfg):
+    _say("gemm", dtype, R, E, Kd, N, cname, cfg)
+    g = torch.Generator().manual_seed(R + E + Kd + N)
+    counts = _ragged_counts(cname, R, E, g)
+    cs = counts.cumsum(0)
+    offs = _offsets(counts, gpu_device)
+    A = torch.randn(R, Kd, generator=g).to(dtype)
+    B = (torch.randn(E, Kd, N, generator=g) * 0.1).to(dtype)
+    d = gpu_device
+    tol = 4e-3 if dtype == torch.bfloat16 else F32_TOL
+
+    # NN: C = A @ B[e]
+    C = ops.grouped_gemm_nn(A.to(d), B.to(d), offs, tile_cfg=cfg)
+    ref = O.grouped_gemm(A.double(), B.double(), cs)
+    assert O.rel_l2(C.cpu(), ref) <= tol, "nn"
+
+    # NN with the row gather folded in
+    if dtype == torch.bfloat16 or True:
+        Tn = max(R // 2, 1)
+        src = torch.randn(Tn, Kd, generator=g).to(dtype)
+        rmap = torch.randint(0, Tn, (R,), generator=g)
+        C2 = ops.grouped_gemm_nn(src.to(d), B.to(d), offs, a_row_map=rmap.to(torch.int32).to(d), tile_cfg=cfg)
+        ref2 = O.grouped_gemm(src.double()[rmap], B.double(), cs)
+        assert O.rel_l2(C2.cpu(), ref2) <= tol, "nn + row map"
+
+    # NT: D = G @ B[e]^T
+    G = torch.randn(R, N, generator=g).to(dtype)
+    if dtype == torch.float32 or (N % 64 == 0 and Kd % 8 == 0):
+        D = ops.grouped_gemm_nt(G.to(d), B.to(d), offs, tile_cfg=cfg)
+        refD = O.grouped_gemm(G.double(), B.double().transpose(1, 2).contiguous(), cs)
+        assert O.rel_l2(D.cpu(), refD) <= tol, "nt"
+
+    # wgrad: W[e] = A_e^T @ G_e, zeros for empty experts
+    W = ops.grouped_gemm_wgrad(A.to(d), G.to(d), offs, E, tile_cfg=cfg)
+    refW = torch.zeros(E, Kd, N, dtype=torch.float64)
+    start = 0
+    for e in range(E):
+        end = int(cs[e])
+        refW[e] = A.double()[start:end].t() @ G.double()[start:end]
+        start = end
+    assert O.rel_l2(W.cpu(), refW) <= tol, "wgrad"
+    for e in range(E):
+        if int(counts[e]) == 0:
+            assert bool((W[e] == 0).all()), "empty expert must produce exact zeros"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("cfg", [0, 1, 3])
+@pytest.mark.parametrize("act", ["silu", "gpt_oss"])
+def test_gateup_activation_fused(ops, gpu_device, dtype, cfg, act):
+    _say("gateup", dtype, cfg, act)
+    code = {"silu": 0, "gelu": 1, "relu": 2, "gpt_oss": 3}[act]
+    g = torch.Generator().manual_seed(17)
+    R, E, H, I = 900, 5, 128, 96
+    counts = _ragged_counts("ragged", R, E, g)
+    offs = _offsets(counts, gpu_device)
+    xp = torch.randn(R, H, generator=g).to(dtype)
+    w = (torch.randn(E, H, 2 * I, generator=g) * 0.1).to(dtype)
+    gu, inter = ops.grouped_gemm_gateup_act_fwd(xp.to(gpu_device), w.to(gpu_device), offs, code, tile_cfg=cfg)
+    ref_gu = O.grouped_gemm(xp.double(), w.double(), counts.cumsum(0))
+    tol = 4e-3 if dtype == torch.bfloat16 else F32_TOL
+    assert O.rel_l2(gu.cpu(), ref_gu) <= tol
+    ref_inter = ref_gu[:, 1::2] * O.activation(act)(ref_gu[:, 0::2])
+    assert O.rel_l2(inter.cpu(), ref_inter) <= (BF16_TOL if dtype == torch.bfloat16 else 2e-5)
+    # inter is exactly the activation of the stored (rounded) gate_up
+    gu_s = gu.cpu().double()
+    chk = gu_s[:, 1::2] * O.activation(act)(gu_s[:, 0::2])
+    assert O.rel_l2(inter.cpu(), chk) <= (4e-3 if dtype == torch.bfloat16 else 2e-6)
+    if dtype == torch.bfloat16:
+        _, inter2 = ops.grouped_gemm_gateup_act_fwd(
+            xp.to(gpu_device), w.to(gpu_device), offs, code, tile_cfg=cfg, want_gate_up=False
+        )
+        assert torch.equal(inter2, inter)
+
+
+def test_grouped_gemm_rows_outside_groups_untouched(ops, gpu_device):
+    """Rows past offsets[E] are never written (the tile map covers only routed rows)."""
+    g = torch.Generator().manual_seed(5)
+    R, E, Kd, N = 640, 4, 64, 128
+    counts = torch.tensor([100, 0, 250, 90])  # 440 of 640 rows in use
+    offs = _offsets(counts, gpu_device)
+    A = torch.randn(R, Kd, generator=g).to(torch.bfloat16).to(gpu_device)
+    B = torch.randn(E, Kd, N, generator=g).to(torch.bfloat16).to(gpu_device)
+    lib_ops = ops
+    C = lib_ops.grouped_gemm_nn(A, B, offs)
+    ref = O.grouped_gemm(A.cpu().double()[:440], B.cpu().double(), counts.cumsum(0))
+    assert O.rel_l2(C[:440].cpu(), ref) <= 4e-3
