@@ -22,12 +22,15 @@
 // routing skew.
 #include "amoe_common.h"
 
+#include <type_traits>
+
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 mfma_bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float mfma_f32x16;
 
 namespace {
 
-constexpr int BK = 64;
+constexpr int BK = 32;      // K extent of one LDS stage
+constexpr int NSTAGE = 4;   // LDS stages in flight
 
 struct GemmArgs {
     const bf16_t* A;
@@ -46,6 +49,8 @@ struct GemmArgs {
     int N;        // output columns
     int n_ntiles;
     int n_mt;     // wgrad mode: M tiles per expert
+    int gm, gn;   // blocks of one XCD work on super-tiles of gm x gn tiles
+    int sn;       // super-tiles along N
 };
 
 enum { EPI_STORE = 0, EPI_GATED = 1 };
@@ -96,6 +101,62 @@ tile_map_kernel(const int32_t* __restrict__ offsets, int E, int bm, int4* __rest
 __device__ __forceinline__ uint32_t perm_lo(uint32_t w1, uint32_t w0) { return __builtin_amdgcn_perm(w1, w0, 0x05040100u); }
 __device__ __forceinline__ uint32_t perm_hi(uint32_t w1, uint32_t w0) { return __builtin_amdgcn_perm(w1, w0, 0x07060302u); }
 
+// 16 zero bytes that masked lanes of a direct-to-LDS load read instead of out-of-range rows
+__device__ __attribute__((aligned(16))) uint32_t g_zero_chunk[4] = {0u, 0u, 0u, 0u};
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// Scheduling hints: ask the backend to build the sequence (n_i x MASK, 1 x MFMA) for
+// i < H, with the TOTAL instructions of class MASK spread evenly over the H MFMAs.
+template <int MASK, int TOTAL, int H, int I = 0>
+__device__ __forceinline__ void sched_interleave()
+{
+    if constexpr (I < H) {
+        constexpr int n = (TOTAL * (I + 1)) / H - (TOTAL * I) / H;
+        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(MASK, n, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        sched_interleave<MASK, TOTAL, H, I + 1>();
+    }
+}
+constexpr int SCHED_VALU = 0x002, SCHED_VMEM = 0x010, SCHED_DS_RD = 0x100;
+
+// wait until at most N of this wave's vector-memory operations (incl. direct-to-LDS loads)
+// are outstanding; the other counters are left alone
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N <= 63, "vmcnt is 6 bits");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// (DS reads in the first half, VMEM spread over all) interleaved with H MFMAs
+template <int NDS, int NVM, int H, int I = 0>
+__device__ __forceinline__ void sched_mix()
+{
+    if constexpr (I < H) {
+        constexpr int HH = H / 2;
+        constexpr int nd = (I < HH) ? (NDS * (I + 1)) / HH - (NDS * I) / HH : 0;
+        if constexpr (nd > 0) __builtin_amdgcn_sched_group_barrier(0x100, nd, 0);
+        constexpr int nv = (NVM * (I + 1)) / H - (NVM * I) / H;
+        if constexpr (nv > 0) __builtin_amdgcn_sched_group_barrier(0x010, nv, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        sched_mix<NDS, NVM, H, I + 1>();
+    }
+}
+// wave-level half of a workgroup barrier for LDS data: this wave's LDS reads have returned and
+// all but N of its loads have landed; then the hardware barrier.  (No memory fence: LDS is not
+// cached and the direct-to-LDS loads are tracked by vmcnt.)
+template <int N>
+__device__ __forceinline__ void lds_barrier()
+{
+    static_assert(N >= 0 && N <= 63, "vmcnt is 6 bits");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+}
+using T_ = std::true_type;
+using F_ = std::false_type;
+
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT>
 __global__ void __launch_bounds__(WGM * WGN * 64)
 grouped_gemm_bf16_kernel(GemmArgs p)
@@ -107,24 +168,33 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     static_assert(TN % 2 == 0, "N tiles come in even/odd pairs");
     static_assert(!WGRAD || (TM % 2 == 0 && !B_KC), "wgrad pairs both operands");
     static_assert(BM >= 128 && BN >= 128, "K-strided swizzle needs 16 chunks per row");
-    constexpr int A_CH = BM * 8, B_CH = BN * 8;   // 16-byte chunks per stage
+    constexpr int A_CH = BM * 4, B_CH = BN * 4;   // 16-byte chunks per stage (a 32-wide K row is 4 chunks)
+    constexpr int STAGE = A_CH + B_CH;
     constexpr int PER_A = A_CH / NT, PER_B = B_CH / NT;
     static_assert(A_CH % NT == 0 && B_CH % NT == 0, "tile must split evenly over the block");
 
     extern __shared__ u32x4_t smem[];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const int lj = lane & 31, lg = lane >> 5;
 
     // ------------------------------------------------------------ block -> tile
+    // Workgroups are dealt to the 8 XCDs round-robin.  The ~32 workgroups resident on one XCD
+    // are made to cover one gm x gn super-tile, so its gm A panels and gn B panels are fetched
+    // into that XCD's L2 once and shared; super-tiles themselves rotate over the XCDs.
     const int b = blockIdx.x;
     const int xcd = b & 7;
     const int q = b >> 3;
-    const int grp = q / p.n_ntiles;
-    const int nt = q - grp * p.n_ntiles;
-    const int pm = grp * 8 + xcd;
+    const int per_super = p.gm * p.gn;
+    const int sid = (q / per_super) * 8 + xcd;
+    const int w = q % per_super;
+    const int sm = sid / p.sn, sn_i = sid - sm * p.sn;
+    const int pm = sm * p.gm + w / p.gn;
+    const int nt = sn_i * p.gn + w % p.gn;
+    if (nt >= p.n_ntiles) return;
     int e, m0, mend, kt_count;
     int r0 = 0, r1 = 0;
     if (!WGRAD) {
@@ -146,8 +216,11 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     const int n0 = nt * BN;
 
     // ------------------------------------------------------------ global load plans
+    // Loads go straight from global memory into LDS: lane l of a wave fills the 16-byte chunk
+    // (wave's base + l), so chunk c = tid + NT*i of a stage is filled by thread tid in its i-th
+    // load.  The XOR swizzle of the LDS layout is applied on the SOURCE side: the thread that
+    // fills physical chunk c fetches the logical chunk that belongs there.
     uint32_t aoff[PER_A], boff[PER_B];
-    int a_lds[PER_A], b_lds[PER_B];
     int a_kr[PER_A], b_kr[PER_B];  // wgrad: k row of the chunk, for the ragged-end mask
     const bf16_t* Ab = p.A;
     const bf16_t* Bb = p.B;
@@ -155,18 +228,16 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     for (int i = 0; i < PER_A; ++i) {
         const int c = tid + NT * i;
         if (A_KC) {
-            const int row = c >> 3, kc = c & 7;
+            const int row = c >> 2, kc = (c & 3) ^ ((row >> 2) & 3);
             int gr = min(m0 + row, mend - 1);
             if (p.a_row_map) gr = p.a_row_map[gr];
             aoff[i] = (uint32_t)gr * (uint32_t)p.lda + kc * 8;
-            a_lds[i] = row * 8 + (kc ^ (row & 7));
             a_kr[i] = 0;
         } else {
             constexpr int CPR = BM / 8;
-            const int krow = c / CPR, mc = c % CPR;
+            const int krow = c / CPR, mc = (c % CPR) ^ (((krow >> 3) & 1) << 3);
             const int col = min(m0 + mc * 8, p.M - 8);
             aoff[i] = (uint32_t)krow * (uint32_t)p.lda + col;
-            a_lds[i] = krow * CPR + (mc ^ (((krow >> 3) & 1) << 3));
             a_kr[i] = krow;
         }
     }
@@ -174,17 +245,18 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     for (int i = 0; i < PER_B; ++i) {
         const int c = tid + NT * i;
         if (B_KC) {
-            const int row = c >> 3, kc = c & 7;
-            const int gn = min(n0 + row, p.N - 1);
+            // LDS row slot s of a 64-row block holds column 2*(s%32) + s/32 of that block, so the
+            // even columns (one MFMA tile) and the odd columns (its partner) are each 32
+            // consecutive LDS rows
+            const int row = c >> 2, kc = (c & 3) ^ ((row >> 2) & 3);
+            const int gn = min(n0 + (row & ~63) + 2 * (row & 31) + ((row >> 5) & 1), p.N - 1);
             boff[i] = (uint32_t)gn * (uint32_t)p.ldb + kc * 8;
-            b_lds[i] = row * 8 + (kc ^ ((row >> 1) & 7));
             b_kr[i] = 0;
         } else {
             constexpr int CPR = BN / 8;
-            const int krow = c / CPR, nc = c % CPR;
+            const int krow = c / CPR, nc = (c % CPR) ^ (((krow >> 3) & 1) << 3);
             const int col = min(n0 + nc * 8, p.N - 8);
             boff[i] = (uint32_t)krow * (uint32_t)p.ldb + col;
-            b_lds[i] = krow * CPR + (nc ^ (((krow >> 3) & 1) << 3));
             b_kr[i] = krow;
         }
     }
@@ -196,43 +268,31 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     }
     const int k_rows = r1 - r0;  // wgrad: rows of this expert
 
-    u32x4_t ra[PER_A], rb[PER_B];
-    auto load_global = [&](int kt) {
+    // wgrad: rows past the end of the expert read a block of zeros instead (only the last K
+    // tile of an expert can be ragged, the select costs two VALU ops per load)
+    auto issue_a = [&](int kt, auto LO, auto HI) {
+        constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
         const int k0 = kt * BK;
+        u32x4_t* sa = smem + (kt & (NSTAGE - 1)) * STAGE + wave * 64;
+        const bf16_t* a_base = A_KC ? Ab + k0 : Ab + (long long)k0 * p.lda;
 #pragma unroll
-        for (int i = 0; i < PER_A; ++i) {
-            if (A_KC) {
-                ra[i] = *reinterpret_cast<const u32x4_t*>(Ab + aoff[i] + k0);
-            } else {
-                const bool ok = k0 + a_kr[i] < k_rows;
-                const bf16_t* src = Ab + (ok ? aoff[i] + (uint32_t)k0 * (uint32_t)p.lda : 0u);
-                u32x4_t v = *reinterpret_cast<const u32x4_t*>(ok ? src : p.A);
-                u32x4_t z = {0u, 0u, 0u, 0u};
-                ra[i] = ok ? v : z;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < PER_B; ++i) {
-            if (B_KC) {
-                rb[i] = *reinterpret_cast<const u32x4_t*>(Bb + boff[i] + k0);
-            } else if (!WGRAD) {
-                rb[i] = *reinterpret_cast<const u32x4_t*>(Bb + boff[i] + (uint32_t)k0 * (uint32_t)p.ldb);
-            } else {
-                const bool ok = k0 + b_kr[i] < k_rows;
-                const bf16_t* src = Bb + (ok ? boff[i] + (uint32_t)k0 * (uint32_t)p.ldb : 0u);
-                u32x4_t v = *reinterpret_cast<const u32x4_t*>(ok ? src : p.B);
-                u32x4_t z = {0u, 0u, 0u, 0u};
-                rb[i] = ok ? v : z;
-            }
+        for (int i = lo; i < hi; ++i) {
+            const bf16_t* src = a_base + aoff[i];
+            if (WGRAD) src = (k0 + a_kr[i] < k_rows) ? src : reinterpret_cast<const bf16_t*>(g_zero_chunk);
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sa + NT * i), 16, 0, 0);
         }
     };
-    auto store_lds = [&](int buf) {
-        u32x4_t* sa = smem + buf * (A_CH + B_CH);
-        u32x4_t* sb = sa + A_CH;
+    auto issue_b = [&](int kt, auto LO, auto HI) {
+        constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
+        const int k0 = kt * BK;
+        u32x4_t* sb = smem + (kt & (NSTAGE - 1)) * STAGE + A_CH + wave * 64;
+        const bf16_t* b_base = B_KC ? Bb + k0 : Bb + (long long)k0 * p.ldb;
 #pragma unroll
-        for (int i = 0; i < PER_A; ++i) sa[a_lds[i]] = ra[i];
-#pragma unroll
-        for (int i = 0; i < PER_B; ++i) sb[b_lds[i]] = rb[i];
+        for (int i = lo; i < hi; ++i) {
+            const bf16_t* src = b_base + boff[i];
+            if (WGRAD) src = (k0 + b_kr[i] < k_rows) ? src : reinterpret_cast<const bf16_t*>(g_zero_chunk);
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sb + NT * i), 16, 0, 0);
+        }
     };
 
     mfma_f32x16 acc[TM][TN];
@@ -244,14 +304,17 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     // ------------------------------------------------------------ fragment readers
-    auto read_a = [&](const u32x4_t* sa, int ks, mfma_bf16x8 (&fa)[TM]) {
+    // "raw" fragments are what comes out of LDS: for a K-contiguous operand the MFMA operand
+    // itself, for a K-strided operand eight dwords per tile pair still to be split by v_perm.
+    constexpr int RAW_A = A_KC ? TM : TM * 2;   // u32x4 registers
+    constexpr int RAW_B = B_KC ? TN : TN * 2;
+    auto read_a = [&](const u32x4_t* sa, int ks, u32x4_t (&ra)[RAW_A]) {
         if (A_KC) {
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
                 const int row = wm * WTM + t * 32 + lj;
                 const int kc = ks * 2 + lg;
-                u32x4_t v = sa[row * 8 + (kc ^ (row & 7))];
-                fa[t] = __builtin_bit_cast(mfma_bf16x8, v);
+                ra[t] = sa[row * 4 + (kc ^ ((row >> 2) & 3))];
             }
         } else {
             constexpr int CPR = BM / 8;
@@ -260,27 +323,21 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             for (int pr = 0; pr < TM / 2; ++pr) {
                 const int word = (wm * WTM + pr * 64) / 2 + lj;
                 const int chunk = (word >> 2) ^ (lg << 3);
-                uint32_t w[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int krow = ks * 16 + lg * 8 + i;
-                    w[i] = sw[(krow * CPR + chunk) * 4 + (word & 3)];
+                    ra[pr * 2 + (i >> 2)][i & 3] = sw[(krow * CPR + chunk) * 4 + (word & 3)];
                 }
-                u32x4_t lo = {perm_lo(w[1], w[0]), perm_lo(w[3], w[2]), perm_lo(w[5], w[4]), perm_lo(w[7], w[6])};
-                u32x4_t hi = {perm_hi(w[1], w[0]), perm_hi(w[3], w[2]), perm_hi(w[5], w[4]), perm_hi(w[7], w[6])};
-                fa[2 * pr] = __builtin_bit_cast(mfma_bf16x8, lo);
-                fa[2 * pr + 1] = __builtin_bit_cast(mfma_bf16x8, hi);
             }
         }
     };
-    auto read_b = [&](const u32x4_t* sb, int ks, mfma_bf16x8 (&fb)[TN]) {
+    auto read_b = [&](const u32x4_t* sb, int ks, u32x4_t (&rb)[RAW_B]) {
         if (B_KC) {
 #pragma unroll
             for (int t = 0; t < TN; ++t) {
-                const int row = wn * WTN + (t >> 1) * 64 + 2 * lj + (t & 1);
+                const int row = wn * WTN + t * 32 + lj;
                 const int kc = ks * 2 + lg;
-                u32x4_t v = sb[row * 8 + (kc ^ ((row >> 1) & 7))];
-                fb[t] = __builtin_bit_cast(mfma_bf16x8, v);
+                rb[t] = sb[row * 4 + (kc ^ ((row >> 2) & 3))];
             }
         } else {
             constexpr int CPR = BN / 8;
@@ -289,45 +346,153 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             for (int pr = 0; pr < TN / 2; ++pr) {
                 const int word = (wn * WTN + pr * 64) / 2 + lj;
                 const int chunk = (word >> 2) ^ (lg << 3);
-                uint32_t w[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int krow = ks * 16 + lg * 8 + i;
-                    w[i] = sw[(krow * CPR + chunk) * 4 + (word & 3)];
+                    rb[pr * 2 + (i >> 2)][i & 3] = sw[(krow * CPR + chunk) * 4 + (word & 3)];
                 }
-                u32x4_t lo = {perm_lo(w[1], w[0]), perm_lo(w[3], w[2]), perm_lo(w[5], w[4]), perm_lo(w[7], w[6])};
-                u32x4_t hi = {perm_hi(w[1], w[0]), perm_hi(w[3], w[2]), perm_hi(w[5], w[4]), perm_hi(w[7], w[6])};
-                fb[2 * pr] = __builtin_bit_cast(mfma_bf16x8, lo);
-                fb[2 * pr + 1] = __builtin_bit_cast(mfma_bf16x8, hi);
             }
+        }
+    };
+    // raw -> MFMA operands (identity for K-contiguous operands)
+    auto to_frag_pair = [&](const u32x4_t& w03, const u32x4_t& w47, mfma_bf16x8& even, mfma_bf16x8& odd) {
+        u32x4_t lo = {perm_lo(w03[1], w03[0]), perm_lo(w03[3], w03[2]), perm_lo(w47[1], w47[0]), perm_lo(w47[3], w47[2])};
+        u32x4_t hi = {perm_hi(w03[1], w03[0]), perm_hi(w03[3], w03[2]), perm_hi(w47[1], w47[0]), perm_hi(w47[3], w47[2])};
+        even = __builtin_bit_cast(mfma_bf16x8, lo);
+        odd = __builtin_bit_cast(mfma_bf16x8, hi);
+    };
+    auto make_fa = [&](const u32x4_t (&ra)[RAW_A], mfma_bf16x8 (&fa)[TM]) {
+        if (A_KC) {
+#pragma unroll
+            for (int t = 0; t < TM; ++t) fa[t] = __builtin_bit_cast(mfma_bf16x8, ra[t]);
+        } else {
+#pragma unroll
+            for (int pr = 0; pr < TM / 2; ++pr) to_frag_pair(ra[2 * pr], ra[2 * pr + 1], fa[2 * pr], fa[2 * pr + 1]);
+        }
+    };
+    auto make_fb = [&](const u32x4_t (&rb)[RAW_B], mfma_bf16x8 (&fb)[TN]) {
+        if (B_KC) {
+#pragma unroll
+            for (int t = 0; t < TN; ++t) fb[t] = __builtin_bit_cast(mfma_bf16x8, rb[t]);
+        } else {
+#pragma unroll
+            for (int pr = 0; pr < TN / 2; ++pr) to_frag_pair(rb[2 * pr], rb[2 * pr + 1], fb[2 * pr], fb[2 * pr + 1]);
+        }
+    };
+    // quarter Q of a K step's MFMAs (A tile outer, B tile inner)
+    constexpr int N_MFMA = TM * TN;
+    static_assert(N_MFMA % 4 == 0, "a K step is issued in four chunks");
+    auto mma_quarter = [&](const mfma_bf16x8 (&fa)[TM], const mfma_bf16x8 (&fb)[TN], auto Q) {
+        constexpr int q = decltype(Q)::value;
+#pragma unroll
+        for (int f = q * (N_MFMA / 4); f < (q + 1) * (N_MFMA / 4); ++f) {
+            const int i = f / TN, j = f % TN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
     };
 
     // ------------------------------------------------------------ main loop
-    if (kt_count > 0) {
-        load_global(0);
-        store_lds(0);
-    }
-    __syncthreads();
-    for (int kt = 0; kt < kt_count; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < kt_count;
-        if (more) load_global(kt + 1);
-        const u32x4_t* sa = smem + cur * (A_CH + B_CH);
-        const u32x4_t* sb = sa + A_CH;
+    // NSTAGE = 4 LDS stages of one 32-wide K tile each (two MFMA K steps).  Iteration j works
+    // on tile j (stage j % 4):
+    //   step A: MFMAs on the ks=0 fragments | fetch the ks=1 fragments of tile j
+    //           | issue the B half of the loads of tile j+3
+    //   wait until tile j+1 has landed (the loads of tiles j+2, j+3 may stay in flight), barrier:
+    //           tile j+1 is visible and stage j % 4 is free (every wave holds its last fragments)
+    //   step B: MFMAs on the ks=1 fragments | fetch the ks=0 fragments of tile j+1
+    //           | issue the A half of the loads of tile j+4 into the stage just freed
+    // so the direct-to-LDS loads trickle out evenly (the L1 path moves 64 bytes a clock, half of
+    // what the MFMAs consume at full rate) and each has about two iterations to land.
+    // A step is written as four chunks fenced by scheduling barriers, each pairing a quarter of
+    // the MFMAs with one kind of side work: A-fragment reads, B-fragment reads, loads, loads +
+    // the v_perm splitting of K-strided fragments for the next step.
+    constexpr int PER = PER_A + PER_B;
+    static_assert(2 * PER + PER_A <= 63, "vmcnt is a 6-bit counter");
+    using IC0 = std::integral_constant<int, 0>;
+    using IC1 = std::integral_constant<int, 1>;
+    using IC2 = std::integral_constant<int, 2>;
+    using IC3 = std::integral_constant<int, 3>;
+    using A_HALF = std::integral_constant<int, (PER_A + 1) / 2>;
+    using A_ALL = std::integral_constant<int, PER_A>;
+    using B_HALF = std::integral_constant<int, (PER_B + 1) / 2>;
+    using B_ALL = std::integral_constant<int, PER_B>;
+    u32x4_t ra[RAW_A], rb[RAW_B];
+    mfma_bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+
+    // prologue: tiles 0..2 and the A half of tile 3 go out, tile 0 is awaited
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            mfma_bf16x8 fa[TM], fb[TN];
-            read_a(sa, ks, fa);
-            read_b(sb, ks, fb);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    for (int t = 0; t < NSTAGE - 1; ++t) {
+        if (t < kt_count) {
+            issue_a(t, IC0{}, A_ALL{});
+            issue_b(t, IC0{}, B_ALL{});
         }
-        if (more) store_lds(cur ^ 1);
-        __syncthreads();
+    }
+    if (kt_count > NSTAGE - 1) {
+        issue_a(NSTAGE - 1, IC0{}, A_ALL{});
+        lds_barrier<2 * PER + PER_A>();
+    } else {
+        lds_barrier<0>();
+    }
+    if (kt_count > 0) {
+        read_a(smem, 0, ra);
+        read_b(smem + A_CH, 0, rb);
+        make_fa(ra, fa0);
+        make_fb(rb, fb0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // LOAD_B: tile kt+3 exists; LOAD_A: tile kt+4 exists; WAITN: loads younger than tile kt+1
+    auto k_tile = [&](auto LOAD_B, auto LOAD_A, auto WAITN, auto NEXT, int kt) {
+        constexpr bool load_b = decltype(LOAD_B)::value, load_a = decltype(LOAD_A)::value;
+        constexpr bool next = decltype(NEXT)::value;
+        constexpr int waitn = decltype(WAITN)::value;
+        const u32x4_t* sa = smem + (kt & (NSTAGE - 1)) * STAGE;
+        const u32x4_t* sb = sa + A_CH;
+        // ---- step A: MFMAs on (fa0, fb0)
+        read_a(sa, 1, ra);
+        mma_quarter(fa0, fb0, IC0{});
+        __builtin_amdgcn_sched_barrier(0);
+        read_b(sb, 1, rb);
+        mma_quarter(fa0, fb0, IC1{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (load_b) issue_b(kt + 3, IC0{}, B_HALF{});
+        mma_quarter(fa0, fb0, IC2{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (load_b) issue_b(kt + 3, B_HALF{}, B_ALL{});
+        make_fa(ra, fa1);
+        make_fb(rb, fb1);
+        mma_quarter(fa0, fb0, IC3{});
+        __builtin_amdgcn_sched_barrier(0);
+        lds_barrier<waitn>();
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- step B: MFMAs on (fa1, fb1)
+        const u32x4_t* na = smem + ((kt + 1) & (NSTAGE - 1)) * STAGE;
+        if (next) read_a(na, 0, ra);
+        mma_quarter(fa1, fb1, IC0{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (next) read_b(na + A_CH, 0, rb);
+        mma_quarter(fa1, fb1, IC1{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (load_a) issue_a(kt + 4, IC0{}, A_HALF{});
+        mma_quarter(fa1, fb1, IC2{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (load_a) issue_a(kt + 4, A_HALF{}, A_ALL{});
+        if (next) {
+            make_fa(ra, fa0);
+            make_fb(rb, fb0);
+        }
+        mma_quarter(fa1, fb1, IC3{});
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    {
+        using W0 = std::integral_constant<int, 0>;
+        using W1 = std::integral_constant<int, PER>;
+        using W2 = std::integral_constant<int, 2 * PER>;
+        int kt = 0;
+        for (; kt + 4 < kt_count; ++kt) k_tile(T_{}, T_{}, W2{}, T_{}, kt);
+        if (kt + 4 == kt_count) { k_tile(T_{}, F_{}, W2{}, T_{}, kt); ++kt; }
+        if (kt + 3 == kt_count) { k_tile(F_{}, F_{}, W1{}, T_{}, kt); ++kt; }
+        if (kt + 2 == kt_count) { k_tile(F_{}, F_{}, W0{}, T_{}, kt); ++kt; }
+        if (kt + 1 == kt_count) k_tile(F_{}, F_{}, W0{}, F_{}, kt);
     }
 
     // ------------------------------------------------------------ epilogue
@@ -378,7 +543,7 @@ template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int A
 int launch_cfg(const GemmArgs& a, int grid, hipStream_t s)
 {
     auto kern = grouped_gemm_bf16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT>;
-    constexpr int lds_bytes = 2 * (BM + BN) * BK * 2;
+    constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -403,6 +568,8 @@ inline TileCfg pick_cfg(int tile_cfg)
         case 1: return {128, 128};
         case 2: return {256, 128};
         case 3: return {256, 256};
+        case 4: return {256, 256};
+        case 5: return {256, 256};
         default: return {256, 128};
     }
 }
@@ -413,11 +580,26 @@ int launch_any(const GemmArgs& a, int tile_cfg, int grid, hipStream_t s)
     switch (tile_cfg) {
         case 1: return launch_cfg<128, 128, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
         case 3: return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
+        case 4: return launch_cfg<256, 256, 2, 4, A_KC, B_KC, EPI, ACT>(a, grid, s);
+        case 5: return launch_cfg<256, 256, 4, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
         default: return launch_cfg<256, 128, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
     }
 }
 
 }  // namespace
+
+// super-tile shape and grid size for `m_tiles` (upper bound) x `n_ntiles` tiles
+static int set_supertiles(GemmArgs& a, long long m_tiles, long long* grid)
+{
+    a.gn = a.n_ntiles < 8 ? a.n_ntiles : 8;
+    a.gm = 32 / a.gn;
+    a.sn = (a.n_ntiles + a.gn - 1) / a.gn;
+    const long long sm = (m_tiles + a.gm - 1) / a.gm;
+    const long long supers = sm * a.sn;
+    *grid = 8 * ((supers + 7) / 8) * a.gm * a.gn;
+    AMOE_REQUIRE(*grid < (1ll << 31), AMOE_ERR_UNSUPPORTED, "grouped_gemm: grid too large");
+    return AMOE_OK;
+}
 
 // workspace: [0,16) tile count, then one int4 per M tile for the smallest tile height (64)
 static inline int ws_max_mtiles(int R, int E, int bm) { return R / bm + E + 1; }
@@ -472,8 +654,10 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
     a.N = N;
     a.n_ntiles = (N + tc.bn - 1) / tc.bn;
     a.n_mt = 0;
-    const int grid = 8 * ((max_mtiles + 7) / 8) * a.n_ntiles;
-    return launch_any<true, B_KC, EPI, ACT>(a, tile_cfg, grid, s);
+    long long grid = 0;
+    rc = set_supertiles(a, max_mtiles, &grid);
+    if (rc) return rc;
+    return launch_any<true, B_KC, EPI, ACT>(a, tile_cfg, (int)grid, s);
 }
 
 int amoe_bf16_gateup_act(const void* xp, const int32_t* a_row_map, const void* w, const int32_t* offsets, void* gate_up,
@@ -519,8 +703,8 @@ int amoe_bf16_wgrad(const void* A, const void* B, const int32_t* offsets, void* 
     a.N = N;
     a.n_ntiles = (N + tc.bn - 1) / tc.bn;
     a.n_mt = (Kd + tc.bm - 1) / tc.bm;
-    const long long pm_total = (long long)E * a.n_mt;
-    const long long grid = 8 * ((pm_total + 7) / 8) * a.n_ntiles;
-    AMOE_REQUIRE(grid < (1ll << 31), AMOE_ERR_UNSUPPORTED, "grouped_gemm_wgrad: grid too large");
+    long long grid = 0;
+    int rc = set_supertiles(a, (long long)E * a.n_mt, &grid);
+    if (rc) return rc;
     return launch_any<false, false, EPI_STORE, 0>(a, tile_cfg, (int)grid, s);
 }

@@ -243,6 +243,10 @@ GEMM_CASES = [
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 1),
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 2),
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 3),
+    (torch.bfloat16, 1000, 8, 128, 192, "ragged", 4),
+    (torch.bfloat16, 1000, 8, 128, 192, "ragged", 5),
+    (torch.bfloat16, 3000, 5, 320, 576, "ragged", 4),
+    (torch.bfloat16, 3000, 5, 320, 576, "holes", 5),
     (torch.bfloat16, 777, 6, 256, 320, "holes", 0),
     (torch.bfloat16, 2500, 16, 512, 384, "ragged", 0),
     (torch.bfloat16, 300, 3, 192, 1096, "ragged", 0),
@@ -300,7 +304,7 @@ def test_grouped_gemm_nn_nt_wgrad(ops, gpu_device, dtype, R, E, Kd, N, cname, cf
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("cfg", [0, 1, 3])
+@pytest.mark.parametrize("cfg", [0, 1, 3, 4, 5])
 @pytest.mark.parametrize("act", ["silu", "gpt_oss"])
 def test_gateup_activation_fused(ops, gpu_device, dtype, cfg, act):
     _say("gateup", dtype, cfg, act)
