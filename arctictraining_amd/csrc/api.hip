@@ -53,7 +53,7 @@ int check_gemm_common(const char* what, int dtype, int R, int E, int d0, int d1,
 int check_gemm_dims(const char* what, int dtype, int red, int other)
 {
     if (dtype == AMOE_BF16) {
-        AMOE_REQUIRE(red % 64 == 0, AMOE_ERR_UNSUPPORTED, "%s: bf16 reduction length %d must be a multiple of 64", what,
+        AMOE_REQUIRE(red % 32 == 0, AMOE_ERR_UNSUPPORTED, "%s: bf16 reduction length %d must be a multiple of 32", what,
                      red);
         AMOE_REQUIRE(other % 8 == 0, AMOE_ERR_UNSUPPORTED, "%s: bf16 extent %d must be a multiple of 8", what, other);
     } else {

@@ -5,9 +5,13 @@
 //   rows / NT   C[rows_e,:] = A[rows_e,:] @ B[e]^T      (data gradient; B is [N',Kd'] so both K-contiguous)
 //   wgrad / TN  C[e] = A[rows_e,:]^T @ B[rows_e,:]      (weight gradient; the reduction runs over the ragged rows)
 //
-// Tiles of BM x BN x 64 are staged through LDS (double buffered, one barrier per K step) by
-// 16-byte global loads; fragments are read back with
-//   * ds_read_b128 when the operand is K-contiguous in LDS (XOR-swizzled 16-byte chunks), or
+// Tiles of BM x BN x 32 move from global memory straight into LDS (global_load_lds, 16 bytes
+// per lane, four stages in flight); the XOR swizzle of the LDS layout is applied on the source
+// side.  Fragments are read back with
+//   * ds_read_b128 when the operand is K-contiguous in LDS.  A 32-wide K row is 4 chunks of
+//     16 bytes; chunk kc of row r sits at position kc ^ ((r >> 2) & 3), which makes the 32
+//     rows a half-wave reads cover every group of 4 banks exactly twice and the 4 lanes of
+//     each quad distinct groups: conflict-free on the 64-bank LDS of gfx950;
 //   * eight ds_read_b32 + v_perm when it is K-strided: a dword holds two ADJACENT columns of
 //     one k row, so one set of reads feeds a PAIR of MFMA tiles, one taking the even and one
 //     the odd columns.  The pair's accumulators then hold (col 2j, col 2j+1) in the same lane
@@ -16,10 +20,10 @@
 //
 // Row-grouped launches take their (expert, first row, end row) per M tile from a tile map
 // that a small kernel builds on the device from the expert offsets: no host sync, empty
-// experts simply own no tile.  Blocks are dealt to the 8 XCDs so that all N tiles of one M
-// tile run on the same XCD (shared A rows and expert weights in that XCD's L2) while
-// consecutive M tiles rotate over XCDs, which keeps the XCDs evenly loaded whatever the
-// routing skew.
+// experts simply own no tile.  Workgroups are dealt to the 8 XCDs so that the ~32 resident on
+// one XCD cover one super-tile of gm x gn tiles (shared A and B panels in that XCD's L2),
+// and super-tiles rotate over the XCDs, which keeps them evenly loaded whatever the routing
+// skew.
 #include "amoe_common.h"
 
 #include <type_traits>
@@ -107,43 +111,6 @@ __device__ __attribute__((aligned(16))) uint32_t g_zero_chunk[4] = {0u, 0u, 0u, 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-// Scheduling hints: ask the backend to build the sequence (n_i x MASK, 1 x MFMA) for
-// i < H, with the TOTAL instructions of class MASK spread evenly over the H MFMAs.
-template <int MASK, int TOTAL, int H, int I = 0>
-__device__ __forceinline__ void sched_interleave()
-{
-    if constexpr (I < H) {
-        constexpr int n = (TOTAL * (I + 1)) / H - (TOTAL * I) / H;
-        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(MASK, n, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        sched_interleave<MASK, TOTAL, H, I + 1>();
-    }
-}
-constexpr int SCHED_VALU = 0x002, SCHED_VMEM = 0x010, SCHED_DS_RD = 0x100;
-
-// wait until at most N of this wave's vector-memory operations (incl. direct-to-LDS loads)
-// are outstanding; the other counters are left alone
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N <= 63, "vmcnt is 6 bits");
-    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-
-// (DS reads in the first half, VMEM spread over all) interleaved with H MFMAs
-template <int NDS, int NVM, int H, int I = 0>
-__device__ __forceinline__ void sched_mix()
-{
-    if constexpr (I < H) {
-        constexpr int HH = H / 2;
-        constexpr int nd = (I < HH) ? (NDS * (I + 1)) / HH - (NDS * I) / HH : 0;
-        if constexpr (nd > 0) __builtin_amdgcn_sched_group_barrier(0x100, nd, 0);
-        constexpr int nv = (NVM * (I + 1)) / H - (NVM * I) / H;
-        if constexpr (nv > 0) __builtin_amdgcn_sched_group_barrier(0x010, nv, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        sched_mix<NDS, NVM, H, I + 1>();
-    }
-}
 // wave-level half of a workgroup barrier for LDS data: this wave's LDS reads have returned and
 // all but N of its loads have landed; then the hardware barrier.  (No memory fence: LDS is not
 // cached and the direct-to-LDS loads are tracked by vmcnt.)
@@ -570,7 +537,7 @@ inline TileCfg pick_cfg(int tile_cfg)
         case 3: return {256, 256};
         case 4: return {256, 256};
         case 5: return {256, 256};
-        default: return {256, 128};
+        default: return {256, 256};
     }
 }
 
@@ -582,7 +549,8 @@ int launch_any(const GemmArgs& a, int tile_cfg, int grid, hipStream_t s)
         case 3: return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
         case 4: return launch_cfg<256, 256, 2, 4, A_KC, B_KC, EPI, ACT>(a, grid, s);
         case 5: return launch_cfg<256, 256, 4, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
-        default: return launch_cfg<256, 128, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
+        case 2: return launch_cfg<256, 128, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
+        default: return launch_cfg<256, 256, 2, 4, A_KC, B_KC, EPI, ACT>(a, grid, s);  // 8 waves, 128x64 per wave
     }
 }
 

@@ -10,7 +10,7 @@
 
 namespace {
 
-constexpr int kChunk = 1024;        // flat slots per wavefront
+constexpr int kChunk = 512;         // flat slots per wavefront
 constexpr int kWavesPerBlock = 4;   // independent chunks per block
 
 __device__ __forceinline__ int load_expert(const int32_t* assign, int f, int T, int K, int E)
@@ -40,33 +40,51 @@ permute_hist_kernel(const int32_t* __restrict__ assign, int T, int K, int E, int
         for (int e = lane; e < E; e += 64) chunk_counts[(size_t)c * E + e] = cnt[w][e];
 }
 
-// one block of 512 threads: thread e owns expert e
-__global__ void __launch_bounds__(AMOE_MAX_EXPERTS)
+// One block of 1024 threads: with EP = E rounded up to a power of two, thread t works for
+// expert t % EP on the (t / EP)-th slice of the chunks, so that the walk over chunks (the only
+// sequential part) is 1024 / EP ways parallel and every load is coalesced over experts.
+constexpr int kScanThreads = 1024;
+
+__global__ void __launch_bounds__(kScanThreads)
 permute_scan_kernel(int32_t* __restrict__ chunk_counts /* in: counts, out: exclusive base inside expert */,
-                    int E, int n_chunks, int32_t* __restrict__ counts, int32_t* __restrict__ offsets)
+                    int E, int EP, int n_chunks, int32_t* __restrict__ counts, int32_t* __restrict__ offsets)
 {
+    __shared__ int32_t part[kScanThreads];       // [slice][EP]
     __shared__ int32_t tot[AMOE_MAX_EXPERTS];
-    const int e = threadIdx.x;
+    const int t = threadIdx.x;
+    const int e = t & (EP - 1);
+    const int g = t / EP;
+    const int G = kScanThreads / EP;
+    const int per = (n_chunks + G - 1) / G;
+    const int c0 = min(g * per, n_chunks), c1 = min(c0 + per, n_chunks);
+    int sum = 0;
+    if (e < E)
+        for (int c = c0; c < c1; ++c) sum += chunk_counts[(size_t)c * E + e];
+    part[t] = sum;
+    __syncthreads();
     int run = 0;
-    if (e < E) {
-        for (int c = 0; c < n_chunks; ++c) {
+    for (int gg = 0; gg < g; ++gg) run += part[gg * EP + e];
+    if (g == G - 1 && e < E) {
+        counts[e] = run + sum;
+        tot[e] = run + sum;
+    }
+    if (e < E)
+        for (int c = c0; c < c1; ++c) {
             int v = chunk_counts[(size_t)c * E + e];
             chunk_counts[(size_t)c * E + e] = run;
             run += v;
         }
-        counts[e] = run;
-    }
-    tot[e] = (e < E) ? run : 0;
+    if (t < AMOE_MAX_EXPERTS && t >= E) tot[t] = 0;
     __syncthreads();
     // Hillis-Steele inclusive scan over experts
     for (int o = 1; o < AMOE_MAX_EXPERTS; o <<= 1) {
-        int add = (e >= o) ? tot[e - o] : 0;
+        int add = (t < AMOE_MAX_EXPERTS && t >= o) ? tot[t - o] : 0;
         __syncthreads();
-        tot[e] += add;
+        if (t < AMOE_MAX_EXPERTS) tot[t] += add;
         __syncthreads();
     }
-    if (e < E) offsets[e + 1] = tot[e];
-    if (e == 0) offsets[0] = 0;
+    if (t < E) offsets[t + 1] = tot[t];
+    if (t == 0) offsets[0] = 0;
 }
 
 __global__ void __launch_bounds__(kWavesPerBlock * AMOE_WAVE)
@@ -139,7 +157,9 @@ AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, int T, int K, int E, in
     int32_t* cc = (int32_t*)workspace;
     hipLaunchKernelGGL(permute_hist_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E, R,
                        n_chunks, cc);
-    hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(AMOE_MAX_EXPERTS), 0, s, cc, E, n_chunks, counts, offsets);
+    int EP = 1;
+    while (EP < E) EP <<= 1;
+    hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, cc, E, EP, n_chunks, counts, offsets);
     hipLaunchKernelGGL(permute_scatter_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E,
                        R, n_chunks, cc, offsets, token_of, slot_of, row_of);
     return amoe_check_launch("permute_plan");

@@ -82,6 +82,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0)
     ap.add_argument("--kernel-iters", type=int, default=10)
+    ap.add_argument("--only-kernels", action="store_true",
+                    help="skip the timed layer steps and the CPU baseline: run each kernel --kernel-iters times "
+                         "(for counter collection), preceded by one plain 1 GiB device copy as a traffic yardstick")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the expert layer on ONE GPU; --gpus must be 1 (no multi-GPU path in this build)")
@@ -119,6 +122,13 @@ def main():
         y = layer(xg)
         y.backward(dyg)
 
+    if args.only_kernels:
+        args.warmup, args.steps, args.no_cpu_baseline = 1, 1, True
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # the yardstick: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -151,6 +161,18 @@ def main():
     es = 2 if dtype == torch.bfloat16 else 4
     it = args.kernel_iters
     c = args.tile_cfg
+    # the kernel symbol (template instance) each launch resolves to: what rocprofv3 reports
+    tile = {1: "128, 128, 2, 2", 2: "256, 128, 2, 2", 3: "256, 256, 2, 2", 5: "256, 256, 4, 2"}.get(c, "256, 256, 2, 4")
+    sym = {
+        "gemm_gateup_act_fwd": f"grouped_gemm_bf16_kernel<{tile}, true, false, 1, 0>",
+        "gemm_down_fwd": f"grouped_gemm_bf16_kernel<{tile}, true, false, 0, 0>",
+        "gemm_dgrad_down": f"grouped_gemm_bf16_kernel<{tile}, true, true, 0, 0>",
+        "gemm_dgrad_gateup": f"grouped_gemm_bf16_kernel<{tile}, true, true, 0, 0>",
+        "gemm_wgrad_down": f"grouped_gemm_bf16_kernel<{tile}, false, false, 0, 0>",
+        "gemm_wgrad_gateup": f"grouped_gemm_bf16_kernel<{tile}, false, false, 0, 0>",
+    }
+    if dtype != torch.bfloat16:
+        sym = {k: "grouped_gemm_f32_kernel" for k in sym}
     # (name, callable, flops per launch, algorithmic bytes per launch)
     kernels = [
         ("gemm_gateup_act_fwd", lambda: ops.grouped_gemm_gateup_act_fwd(xp, wgu_d, offsets, tile_cfg=c), 4.0 * R * H * I,
@@ -185,18 +207,41 @@ def main():
             entry["frac_hbm_peak"] = round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
         entry["_flops"], entry["_bytes"] = flops, nbytes
         breakdown.append(entry)
-    dom = max(breakdown, key=lambda e: e["ms"])
-    if dom["_flops"]:
+    # Roofline of the dominant kernel SYMBOL: the template instance with the largest total time
+    # per step.  The two weight-gradient GEMMs (and the two data-gradient GEMMs) share one
+    # instance, so its figures are launch averages: mean flops per launch / mean duration.
+    groups = {}
+    for e in breakdown:
+        key = sym.get(e["kernel"], e["kernel"])
+        e["symbol"] = key
+        g = groups.setdefault(key, {"ms": 0.0, "flops": 0.0, "bytes": 0.0, "n": 0, "members": []})
+        g["ms"] += e["ms"]
+        g["flops"] += e["_flops"]
+        g["bytes"] += e["_bytes"]
+        g["n"] += 1
+        g["members"].append(e["kernel"])
+    dom_key = max(groups, key=lambda k: groups[k]["ms"])
+    dg = groups[dom_key]
+    avg_ms = dg["ms"] / dg["n"]
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", f"traffic_{args.config}.json")
+    if os.path.exists(tpath):
+        with open(tpath) as fh:
+            traffic = json.load(fh).get(dom_key)
+    if dg["flops"]:
+        ach = dg["flops"] / dg["n"] / (avg_ms * 1e-3) / 1e12
         roofline = {
-            "kernel": dom["kernel"], "bound": "mfma", "achieved": dom["tflops"], "peak": peak, "unit": "TFLOP/s",
-            "frac": round(dom["tflops"] / peak, 4), "traffic": None, "avg_ms": dom["ms"],
-            "flops_per_launch": dom["_flops"],
+            "kernel": dom_key, "launches_per_step": dg["members"], "bound": "mfma", "achieved": round(ach, 1),
+            "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4), "traffic": traffic,
+            "avg_ms": round(avg_ms, 4), "flops_per_launch": dg["flops"] / dg["n"],
+            "algorithmic_bytes_per_launch": dg["bytes"] / dg["n"],
         }
     else:
+        ach = dg["bytes"] / dg["n"] / (avg_ms * 1e-3) / 1e9
         roofline = {
-            "kernel": dom["kernel"], "bound": "hbm", "achieved": dom["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(dom["gbs"] / PEAK_HBM_GBS, 4), "traffic": None, "avg_ms": dom["ms"],
-            "bytes_per_launch": dom["_bytes"],
+            "kernel": dom_key, "launches_per_step": dg["members"], "bound": "hbm", "achieved": round(ach, 1),
+            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": traffic,
+            "avg_ms": round(avg_ms, 4), "bytes_per_launch": dg["bytes"] / dg["n"],
         }
     gemm_ms = sum(e["ms"] for e in breakdown if e["_flops"])
     for e in breakdown:

@@ -255,6 +255,7 @@ def forward(
     compute_dtype: Optional[torch.dtype] = None,
     logits_for_selection: Optional[torch.Tensor] = None,
     replay_assignments: Optional[torch.Tensor] = None,
+    model_dtype: Optional[torch.dtype] = None,
 ) -> Dict[str, torch.Tensor]:
     """moe.py:219-323 on the default path at EP=1, differentiable with autograd.
 
@@ -262,10 +263,11 @@ def forward(
     reference's rounding after each op ("reference rounding" mode: what the
     reference computes on a CPU).  compute_dtype=float32/float64 up-casts the
     (already rounded) inputs once and keeps every intermediate in that type
-    ("exact" mode); the logits are then still rounded through the inputs'
-    dtype, because that rounding decides the routing.
+    ("exact" mode); the logits are then still rounded through the model dtype
+    (`model_dtype`, by default the dtype of x), because that rounding decides
+    the routing.
     """
-    in_dtype = x.dtype
+    in_dtype = model_dtype if model_dtype is not None else x.dtype
     orig_shape = x.shape
     x2d = x.reshape(-1, x.shape[-1])
     if compute_dtype is not None and compute_dtype != in_dtype:
@@ -307,8 +309,12 @@ def forward(
 def forward_backward(x, router_gate, expert_gate_up, expert_down, dy, cfg, **kw):
     """forward + autograd backward with upstream gradient dy.  Gradients are
     returned in the compute dtype (no rounding back to the input dtype)."""
-    leaves = [t.detach().clone().requires_grad_(True) for t in (x, router_gate, expert_gate_up, expert_down)]
-    res = forward(*leaves, cfg, **kw)
+    model_dtype = x.dtype
+    leaf_dtype = kw.get("compute_dtype") or model_dtype
+    leaves = [
+        t.detach().to(leaf_dtype).clone().requires_grad_(True) for t in (x, router_gate, expert_gate_up, expert_down)
+    ]
+    res = forward(*leaves, cfg, model_dtype=model_dtype, **kw)
     y = res["y"]
     y.backward(dy.to(y.dtype).reshape(y.shape))
     res["dx"], res["d_router_gate"], res["d_expert_gate_up"], res["d_expert_down"] = (t.grad for t in leaves)

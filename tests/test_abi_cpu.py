@@ -45,7 +45,7 @@ def test_version_and_error_string(lib):
 
 
 def test_workspace_queries(lib):
-    assert lib.amoe_permute_workspace_bytes(131072, 128) >= (131072 // 1024) * 128 * 4
+    assert lib.amoe_permute_workspace_bytes(131072, 128) >= (131072 // 512) * 128 * 4
     assert lib.amoe_grouped_gemm_workspace_bytes(131072, 128) >= 16 * (131072 // 256 + 128)
     assert lib.amoe_permute_workspace_bytes(0, 8) == 0
 
@@ -85,10 +85,10 @@ def test_row_kernel_argument_errors(lib):
 
 def test_gemm_argument_errors(lib):
     big = 1 << 20
-    # bf16 reduction length must be a multiple of 64
-    assert lib.amoe_grouped_gemm_nn(P, None, P, P, P, 1, 128, 4, 96, 64, P, big, 0, None) == -2
-    assert b"multiple of 64" in lib.amoe_last_error()
-    assert lib.amoe_grouped_gemm_nt(P, None, P, P, P, 1, 128, 4, 64, 96, P, big, 0, None) == -2
+    # bf16 reduction length must be a multiple of 32
+    assert lib.amoe_grouped_gemm_nn(P, None, P, P, P, 1, 128, 4, 48, 64, P, big, 0, None) == -2
+    assert b"multiple of 32" in lib.amoe_last_error()
+    assert lib.amoe_grouped_gemm_nt(P, None, P, P, P, 1, 128, 4, 64, 48, P, big, 0, None) == -2
     assert lib.amoe_grouped_gemm_nn(P, None, P, P, P, 1, 128, 4, 64, 64, P, 8, 0, None) == -3  # workspace
     assert lib.amoe_grouped_gemm_nn(P, None, P, P, P, 1, 128, 4, 64, 64, P, big, 9, None) == -1  # tile_cfg
     assert lib.amoe_grouped_gemm_nn(P, None, None, P, P, 1, 128, 4, 64, 64, P, big, 0, None) == -1
