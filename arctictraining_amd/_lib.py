@@ -27,7 +27,8 @@ SIGNATURES = {
     "amoe_permute_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "amoe_permute_plan": (
         _c_int,
-        [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_size_t, _c_void_p],
+        [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+         _c_void_p, _c_size_t, _c_void_p],
     ),
     "amoe_gather_rows_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p]),
     "amoe_gather_rows_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
@@ -39,7 +40,7 @@ SIGNATURES = {
     "amoe_grouped_gemm_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "amoe_grouped_gemm_gateup_act_fwd": (
         _c_int,
-        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
          _c_void_p, _c_size_t, _c_int, _c_void_p],
     ),
     "amoe_grouped_gemm_nn": (
@@ -56,7 +57,11 @@ SIGNATURES = {
         _c_int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     ),
-    "amoe_gated_act_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
+    "amoe_gated_act_bwd": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_void_p],
+    ),
 }
 
 _lib = None

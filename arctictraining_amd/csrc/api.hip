@@ -19,7 +19,7 @@ AMOE_EXPORT const char* amoe_last_error(void) { return g_err; }
 
 // implemented in gemm_bf16.hip / gemm_f32.hip / rows.hip
 int amoe_bf16_gateup_act(const void* xp, const int32_t* a_row_map, const void* w, const int32_t* offsets, void* gate_up,
-                         void* inter, int R, int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
+                         void* inter, const float* row_scale, int R, int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
                          int tile_cfg, hipStream_t s);
 int amoe_bf16_nn(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                  int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s);
@@ -32,7 +32,8 @@ int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const 
                   hipStream_t s);
 int amoe_f32_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int R, int E, int Kd, int N,
                    hipStream_t s);
-int amoe_launch_gated_act_fwd(const void* gu, void* inter, int dtype, int R, int I, int act, hipStream_t s);
+int amoe_launch_gated_act_fwd(const void* gu, const float* row_scale, void* inter, int dtype, int R, int I, int act,
+                              hipStream_t s);
 
 namespace {
 
@@ -66,7 +67,8 @@ int check_gemm_dims(const char* what, int dtype, int red, int other)
 }  // namespace
 
 AMOE_EXPORT int amoe_grouped_gemm_gateup_act_fwd(const void* xp, const int32_t* a_row_map, const void* w_gate_up,
-                                                 const int32_t* offsets, void* gate_up, void* inter, int dtype, int R,
+                                                 const int32_t* offsets, const float* row_scale, void* gate_up,
+                                                 void* inter, int dtype, int R,
                                                  int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
                                                  int tile_cfg, void* stream)
 {
@@ -83,14 +85,14 @@ AMOE_EXPORT int amoe_grouped_gemm_gateup_act_fwd(const void* xp, const int32_t* 
                  "%s: workspace %zu < %zu bytes", what, workspace_bytes, amoe_grouped_gemm_workspace_bytes(R, E));
     hipStream_t s = (hipStream_t)stream;
     if (dtype == AMOE_BF16)
-        return amoe_bf16_gateup_act(xp, a_row_map, w_gate_up, offsets, gate_up, inter, R, E, H, I, act, workspace,
+        return amoe_bf16_gateup_act(xp, a_row_map, w_gate_up, offsets, gate_up, inter, row_scale, R, E, H, I, act, workspace,
                                     workspace_bytes, tile_cfg, s);
     AMOE_REQUIRE(gate_up, AMOE_ERR_UNSUPPORTED, "%s: the f32 path needs the gate_up buffer", what);
     AMOE_REQUIRE(I % 4 == 0, AMOE_ERR_UNSUPPORTED, "%s: f32 intermediate size %d must be a multiple of 4", what, I);
     rc = amoe_f32_rows(xp, a_row_map, w_gate_up, offsets, gate_up, R, E, H, 2 * I, 2 * I, (long long)H * 2 * I, false,
                        workspace, workspace_bytes, s);
     if (rc) return rc;
-    return amoe_launch_gated_act_fwd(gate_up, inter, dtype, R, I, act, s);
+    return amoe_launch_gated_act_fwd(gate_up, row_scale, inter, dtype, R, I, act, s);
 }
 
 AMOE_EXPORT int amoe_grouped_gemm_nn(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets,

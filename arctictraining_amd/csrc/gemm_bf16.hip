@@ -42,6 +42,7 @@ struct GemmArgs {
     bf16_t* C;
     bf16_t* C2;
     const int32_t* a_row_map;
+    const float* row_scale;  // gated epilogue: inter[r,:] is multiplied by row_scale[r] (null = 1)
     const int32_t* offsets;
     const int4* tile_map;
     const int32_t* n_mtiles;
@@ -470,6 +471,8 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             for (int v = 0; v < 16; ++v) {
                 const int row = m0 + wm * WTM + i * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
                 if (row >= mend) continue;
+                float rs = 1.0f;
+                if (EPI == EPI_GATED && p.row_scale) rs = p.row_scale[row];
 #pragma unroll
                 for (int pr = 0; pr < TN / 2; ++pr) {
                     const int col = n0 + wn * WTN + pr * 64 + 2 * lj;
@@ -478,7 +481,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
                     if (EPI == EPI_GATED) {
                         if (p.C) *reinterpret_cast<uint32_t*>(p.C + (size_t)row * p.ldc + col) = packed;
                         const float gte = bf16_lo(packed), up = bf16_hi(packed);
-                        p.C2[(size_t)row * p.ldc2 + (col >> 1)] = (bf16_t)(up * act_fwd<ACT>(gte));
+                        p.C2[(size_t)row * p.ldc2 + (col >> 1)] = (bf16_t)(rs * up * act_fwd<ACT>(gte));
                     } else {
                         *reinterpret_cast<uint32_t*>(p.C + (size_t)row * p.ldc + col) = packed;
                     }
@@ -595,7 +598,7 @@ int amoe_build_tile_map(const int32_t* offsets, int R, int E, int bm, void* work
 // rows mode driver shared by the three row-grouped entry points
 template <bool B_KC, int EPI, int ACT>
 static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C,
-                         void* C2, int R, int E, int Kred, int N, int ldb, long long strideB, void* workspace,
+                         void* C2, const float* row_scale, int R, int E, int Kred, int N, int ldb, long long strideB, void* workspace,
                          size_t workspace_bytes, int tile_cfg, hipStream_t s)
 {
     TileCfg tc = pick_cfg(tile_cfg);
@@ -609,6 +612,7 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
     a.C = (bf16_t*)C;
     a.C2 = (bf16_t*)C2;
     a.a_row_map = a_row_map;
+    a.row_scale = row_scale;
     a.offsets = offsets;
     a.lda = Kred;
     a.ldb = ldb;
@@ -629,10 +633,10 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
 }
 
 int amoe_bf16_gateup_act(const void* xp, const int32_t* a_row_map, const void* w, const int32_t* offsets, void* gate_up,
-                         void* inter, int R, int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
+                         void* inter, const float* row_scale, int R, int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
                          int tile_cfg, hipStream_t s)
 {
-    AMOE_DISPATCH_ACT(act, return (run_rows_bf16<false, EPI_GATED, ACT>(xp, a_row_map, w, offsets, gate_up, inter, R, E, H,
+    AMOE_DISPATCH_ACT(act, return (run_rows_bf16<false, EPI_GATED, ACT>(xp, a_row_map, w, offsets, gate_up, inter, row_scale, R, E, H,
                                                                         2 * I, 2 * I, (long long)H * 2 * I, workspace,
                                                                         workspace_bytes, tile_cfg, s)))
     return AMOE_ERR_BAD_ARG;
@@ -641,7 +645,7 @@ int amoe_bf16_gateup_act(const void* xp, const int32_t* a_row_map, const void* w
 int amoe_bf16_nn(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                  int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s)
 {
-    return run_rows_bf16<false, EPI_STORE, 0>(A, a_row_map, B, offsets, C, nullptr, R, E, Kd, N, N, (long long)Kd * N,
+    return run_rows_bf16<false, EPI_STORE, 0>(A, a_row_map, B, offsets, C, nullptr, nullptr, R, E, Kd, N, N, (long long)Kd * N,
                                               workspace, workspace_bytes, tile_cfg, s);
 }
 
@@ -649,7 +653,7 @@ int amoe_bf16_nn(const void* A, const int32_t* a_row_map, const void* B, const i
 int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                  int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s)
 {
-    return run_rows_bf16<true, EPI_STORE, 0>(A, a_row_map, B, offsets, C, nullptr, R, E, /*Kred=*/N, /*N out=*/Kd,
+    return run_rows_bf16<true, EPI_STORE, 0>(A, a_row_map, B, offsets, C, nullptr, nullptr, R, E, /*Kred=*/N, /*N out=*/Kd,
                                              /*ldb=*/N, (long long)Kd * N, workspace, workspace_bytes, tile_cfg, s);
 }
 

@@ -90,7 +90,8 @@ permute_scan_kernel(int32_t* __restrict__ chunk_counts /* in: counts, out: exclu
 __global__ void __launch_bounds__(kWavesPerBlock * AMOE_WAVE)
 permute_scatter_kernel(const int32_t* __restrict__ assign, int T, int K, int E, int R, int n_chunks,
                        const int32_t* __restrict__ chunk_base, const int32_t* __restrict__ offsets,
-                       int32_t* __restrict__ token_of, int32_t* __restrict__ slot_of, int32_t* __restrict__ row_of)
+                       const float* __restrict__ scores, int32_t* __restrict__ token_of, int32_t* __restrict__ slot_of,
+                       int32_t* __restrict__ row_of, float* __restrict__ scores_perm)
 {
     __shared__ int32_t run[kWavesPerBlock][AMOE_MAX_EXPERTS];
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -125,6 +126,7 @@ permute_scatter_kernel(const int32_t* __restrict__ assign, int T, int K, int E, 
             token_of[row] = t;
             slot_of[row] = f;
             row_of[(size_t)t * K + k] = row;
+            if (scores_perm) scores_perm[row] = scores[(size_t)t * K + k];
         }
     }
 }
@@ -139,12 +141,13 @@ AMOE_EXPORT size_t amoe_permute_workspace_bytes(int R, int E)
     return (size_t)permute_chunks(R) * (size_t)E * sizeof(int32_t);
 }
 
-AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, int T, int K, int E, int32_t* counts, int32_t* offsets,
-                                  int32_t* token_of, int32_t* slot_of, int32_t* row_of, void* workspace,
-                                  size_t workspace_bytes, void* stream)
+AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                                  int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of,
+                                  float* scores_perm, void* workspace, size_t workspace_bytes, void* stream)
 {
     AMOE_REQUIRE(assign && counts && offsets && token_of && slot_of && row_of && workspace, AMOE_ERR_BAD_ARG,
                  "permute_plan: null pointer");
+    AMOE_REQUIRE(!scores_perm || scores, AMOE_ERR_BAD_ARG, "permute_plan: scores_perm needs scores");
     AMOE_REQUIRE(T > 0 && K > 0 && E > 0, AMOE_ERR_BAD_ARG, "permute_plan: T, K, E must be positive");
     AMOE_REQUIRE(E <= AMOE_MAX_EXPERTS, AMOE_ERR_UNSUPPORTED, "permute_plan: E=%d exceeds %d", E, AMOE_MAX_EXPERTS);
     AMOE_REQUIRE((long long)T * K < (1ll << 31), AMOE_ERR_UNSUPPORTED, "permute_plan: T*K does not fit int32");
@@ -161,6 +164,6 @@ AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, int T, int K, int E, in
     while (EP < E) EP <<= 1;
     hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, cc, E, EP, n_chunks, counts, offsets);
     hipLaunchKernelGGL(permute_scatter_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E,
-                       R, n_chunks, cc, offsets, token_of, slot_of, row_of);
+                       R, n_chunks, cc, offsets, scores, token_of, slot_of, row_of, scores_perm);
     return amoe_check_launch("permute_plan");
 }

@@ -107,45 +107,76 @@ combine_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ out, const in
     }
 }
 
-// inter[r,i] = gu[r,2i+1] * act(gu[r,2i])
+// inter[r,i] = scale[r] * gu[r,2i+1] * act(gu[r,2i])     (one wavefront per row; scale == null -> 1)
 template <typename T, int ACT>
 __global__ void __launch_bounds__(kBlock)
-gated_act_fwd_kernel(const T* __restrict__ gu, T* __restrict__ inter, size_t n_vec_out)
+gated_act_fwd_kernel(const T* __restrict__ gu, const float* __restrict__ scale, T* __restrict__ inter, int R, int I)
 {
     constexpr int V = ElemTraits<T>::kVec;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n_vec_out; i += (size_t)gridDim.x * kBlock) {
-        float a[V], b[V], o[V];
-        ElemTraits<T>::unpack(reinterpret_cast<const u32x4_t*>(gu)[2 * i], a);
-        ElemTraits<T>::unpack(reinterpret_cast<const u32x4_t*>(gu)[2 * i + 1], b);
+    const int lane = threadIdx.x & 63;
+    const int nvec = I / V;
+    for (int r = blockIdx.x * (kBlock / AMOE_WAVE) + (threadIdx.x >> 6); r < R; r += gridDim.x * (kBlock / AMOE_WAVE)) {
+        const float sc = scale ? scale[r] : 1.0f;
+        const u32x4_t* g = reinterpret_cast<const u32x4_t*>(gu + (size_t)r * 2 * I);
+        u32x4_t* o = reinterpret_cast<u32x4_t*>(inter + (size_t)r * I);
+        for (int i = lane; i < nvec; i += AMOE_WAVE) {
+            float a[V], b[V], out[V];
+            ElemTraits<T>::unpack(g[2 * i], a);
+            ElemTraits<T>::unpack(g[2 * i + 1], b);
 #pragma unroll
-        for (int j = 0; j < V / 2; ++j) {
-            o[j] = a[2 * j + 1] * act_fwd<ACT>(a[2 * j]);
-            o[V / 2 + j] = b[2 * j + 1] * act_fwd<ACT>(b[2 * j]);
+            for (int j = 0; j < V / 2; ++j) {
+                out[j] = sc * a[2 * j + 1] * act_fwd<ACT>(a[2 * j]);
+                out[V / 2 + j] = sc * b[2 * j + 1] * act_fwd<ACT>(b[2 * j]);
+            }
+            o[i] = ElemTraits<T>::pack(out);
         }
-        reinterpret_cast<u32x4_t*>(inter)[i] = ElemTraits<T>::pack(o);
     }
 }
 
-// d_gu[r,2i] = d_inter[r,i] * up * act'(gate);  d_gu[r,2i+1] = d_inter[r,i] * act(gate)
+// Backward of inter[r,i] = scale[r] * up * act(gate)   (one wavefront per row):
+//   d_gu[r,2i]   = scale[r] * d_inter[r,i] * up * act'(gate)
+//   d_gu[r,2i+1] = scale[r] * d_inter[r,i] * act(gate)
+//   d_scale[r]   = sum_i d_inter[r,i] * up * act(gate)        written at slot (t,k) of row r
 template <typename T, int ACT>
 __global__ void __launch_bounds__(kBlock)
-gated_act_bwd_kernel(const T* __restrict__ gu, const T* __restrict__ d_inter, T* __restrict__ d_gu, size_t n_vec_inter)
+gated_act_bwd_kernel(const T* __restrict__ gu, const T* __restrict__ d_inter, const float* __restrict__ scale,
+                     const int32_t* __restrict__ slot_of, int n_tokens, int K, T* __restrict__ d_gu,
+                     float* __restrict__ d_scale_tk, int R, int I)
 {
     constexpr int V = ElemTraits<T>::kVec;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n_vec_inter; i += (size_t)gridDim.x * kBlock) {
-        float a[V], b[V], di[V], oa[V], ob[V];
-        ElemTraits<T>::unpack(reinterpret_cast<const u32x4_t*>(gu)[2 * i], a);
-        ElemTraits<T>::unpack(reinterpret_cast<const u32x4_t*>(gu)[2 * i + 1], b);
-        ElemTraits<T>::unpack(reinterpret_cast<const u32x4_t*>(d_inter)[i], di);
+    const int lane = threadIdx.x & 63;
+    const int nvec = I / V;
+    for (int r = blockIdx.x * (kBlock / AMOE_WAVE) + (threadIdx.x >> 6); r < R; r += gridDim.x * (kBlock / AMOE_WAVE)) {
+        const float sc = scale ? scale[r] : 1.0f;
+        const u32x4_t* g = reinterpret_cast<const u32x4_t*>(gu + (size_t)r * 2 * I);
+        const u32x4_t* di = reinterpret_cast<const u32x4_t*>(d_inter + (size_t)r * I);
+        u32x4_t* o = reinterpret_cast<u32x4_t*>(d_gu + (size_t)r * 2 * I);
+        float dot = 0.f;
+        for (int i = lane; i < nvec; i += AMOE_WAVE) {
+            float a[V], b[V], d[V], oa[V], ob[V];
+            ElemTraits<T>::unpack(g[2 * i], a);
+            ElemTraits<T>::unpack(g[2 * i + 1], b);
+            ElemTraits<T>::unpack(di[i], d);
 #pragma unroll
-        for (int j = 0; j < V / 2; ++j) {
-            oa[2 * j] = di[j] * a[2 * j + 1] * act_bwd<ACT>(a[2 * j]);
-            oa[2 * j + 1] = di[j] * act_fwd<ACT>(a[2 * j]);
-            ob[2 * j] = di[V / 2 + j] * b[2 * j + 1] * act_bwd<ACT>(b[2 * j]);
-            ob[2 * j + 1] = di[V / 2 + j] * act_fwd<ACT>(b[2 * j]);
+            for (int j = 0; j < V / 2; ++j) {
+                const float fa = act_fwd<ACT>(a[2 * j]), fb = act_fwd<ACT>(b[2 * j]);
+                dot += d[j] * a[2 * j + 1] * fa + d[V / 2 + j] * b[2 * j + 1] * fb;
+                oa[2 * j] = sc * d[j] * a[2 * j + 1] * act_bwd<ACT>(a[2 * j]);
+                oa[2 * j + 1] = sc * d[j] * fa;
+                ob[2 * j] = sc * d[V / 2 + j] * b[2 * j + 1] * act_bwd<ACT>(b[2 * j]);
+                ob[2 * j + 1] = sc * d[V / 2 + j] * fb;
+            }
+            o[2 * i] = ElemTraits<T>::pack(oa);
+            o[2 * i + 1] = ElemTraits<T>::pack(ob);
         }
-        reinterpret_cast<u32x4_t*>(d_gu)[2 * i] = ElemTraits<T>::pack(oa);
-        reinterpret_cast<u32x4_t*>(d_gu)[2 * i + 1] = ElemTraits<T>::pack(ob);
+        if (d_scale_tk) {
+            dot = wave_sum(dot);
+            if (lane == 0) {
+                const int f = slot_of[r];
+                const int k = f / n_tokens;
+                d_scale_tk[(size_t)(f - k * n_tokens) * K + k] = dot;
+            }
+        }
     }
 }
 
@@ -215,7 +246,7 @@ AMOE_EXPORT int amoe_gather_rows_bwd(const void* d_xp, const int32_t* row_of, co
 AMOE_EXPORT int amoe_combine_fwd(const void* moe_out, const int32_t* row_of, const float* scores, void* y, int dtype,
                                  int T, int K, int H, void* stream)
 {
-    AMOE_REQUIRE(moe_out && row_of && scores && y, AMOE_ERR_BAD_ARG, "combine_fwd: null pointer");
+    AMOE_REQUIRE(moe_out && row_of && y, AMOE_ERR_BAD_ARG, "combine_fwd: null pointer");
     int rc = check_rows("combine_fwd", dtype, T, H);
     if (rc) return rc;
     AMOE_REQUIRE(K > 0 && K <= AMOE_MAX_TOPK, AMOE_ERR_UNSUPPORTED, "combine_fwd: K=%d outside 1..%d", K, AMOE_MAX_TOPK);
@@ -244,41 +275,47 @@ AMOE_EXPORT int amoe_combine_bwd(const void* dy, const void* moe_out, const int3
 }
 
 // used by the f32 gate_up path, which does not fuse the activation into its GEMM
-int amoe_launch_gated_act_fwd(const void* gu, void* inter, int dtype, int R, int I, int act, hipStream_t s)
+int amoe_launch_gated_act_fwd(const void* gu, const float* row_scale, void* inter, int dtype, int R, int I, int act,
+                              hipStream_t s)
 {
-    const int vec = dtype == AMOE_BF16 ? 8 : 4;
-    const size_t n_vec = (size_t)R * I / vec;
-    const int grid = (int)((n_vec + kBlock - 1) / kBlock < 16384 ? (n_vec + kBlock - 1) / kBlock : 16384);
+    const int rows_per_block = kBlock / AMOE_WAVE;
+    const int grid = (R + rows_per_block - 1) / rows_per_block < 65536 ? (R + rows_per_block - 1) / rows_per_block : 65536;
     AMOE_DISPATCH_ACT(act, {
         if (dtype == AMOE_BF16)
             hipLaunchKernelGGL((gated_act_fwd_kernel<bf16_t, ACT>), dim3(grid), dim3(kBlock), 0, s, (const bf16_t*)gu,
-                               (bf16_t*)inter, n_vec);
+                               row_scale, (bf16_t*)inter, R, I);
         else
             hipLaunchKernelGGL((gated_act_fwd_kernel<float, ACT>), dim3(grid), dim3(kBlock), 0, s, (const float*)gu,
-                               (float*)inter, n_vec);
+                               row_scale, (float*)inter, R, I);
     })
     return amoe_check_launch("gated_act_fwd");
 }
 
-AMOE_EXPORT int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, void* d_gate_up, int dtype, int R, int I,
-                                   int act, void* stream)
+AMOE_EXPORT int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, const float* row_scale,
+                                   const int32_t* slot_of, void* d_gate_up, float* d_row_scale, int dtype, int R, int I,
+                                   int T, int K, int act, void* stream)
 {
     AMOE_REQUIRE(gate_up && d_inter && d_gate_up, AMOE_ERR_BAD_ARG, "gated_act_bwd: null pointer");
     int rc = check_rows("gated_act_bwd", dtype, R, I);
     if (rc) return rc;
     AMOE_REQUIRE(act >= AMOE_ACT_SILU && act <= AMOE_ACT_GPT_OSS, AMOE_ERR_BAD_ARG, "gated_act_bwd: bad activation %d",
                  act);
-    const int vec = dtype == AMOE_BF16 ? 8 : 4;
-    const size_t n_vec = (size_t)R * I / vec;
-    const int grid = (int)((n_vec + kBlock - 1) / kBlock < 16384 ? (n_vec + kBlock - 1) / kBlock : 16384);
+    if (d_row_scale) {
+        AMOE_REQUIRE(slot_of, AMOE_ERR_BAD_ARG, "gated_act_bwd: d_row_scale needs slot_of");
+        AMOE_REQUIRE(T > 0 && K > 0 && (long long)T * K == (long long)R, AMOE_ERR_BAD_ARG,
+                     "gated_act_bwd: T*K must equal R (T=%d K=%d R=%d)", T, K, R);
+    }
+    const int rows_per_block = kBlock / AMOE_WAVE;
+    const int grid = (R + rows_per_block - 1) / rows_per_block < 65536 ? (R + rows_per_block - 1) / rows_per_block : 65536;
     hipStream_t s = (hipStream_t)stream;
     AMOE_DISPATCH_ACT(act, {
         if (dtype == AMOE_BF16)
             hipLaunchKernelGGL((gated_act_bwd_kernel<bf16_t, ACT>), dim3(grid), dim3(kBlock), 0, s,
-                               (const bf16_t*)gate_up, (const bf16_t*)d_inter, (bf16_t*)d_gate_up, n_vec);
+                               (const bf16_t*)gate_up, (const bf16_t*)d_inter, row_scale, slot_of, T, K,
+                               (bf16_t*)d_gate_up, d_row_scale, R, I);
         else
             hipLaunchKernelGGL((gated_act_bwd_kernel<float, ACT>), dim3(grid), dim3(kBlock), 0, s, (const float*)gate_up,
-                               (const float*)d_inter, (float*)d_gate_up, n_vec);
+                               (const float*)d_inter, row_scale, slot_of, T, K, (float*)d_gate_up, d_row_scale, R, I);
     })
     return amoe_check_launch("gated_act_bwd");
 }

@@ -106,46 +106,61 @@ class _ExpertLayerFn(torch.autograd.Function):
         logits = torch.matmul(x, router_gate.t())  # plain library GEMM, moe.py:233
         probs, topk_idx, scores = ops.router_topk_fwd(logits, K, opts["normalize"])
         assign = topk_idx if replay is None else replay.to(torch.int32).contiguous()
-        counts, offsets, token_of, slot_of, row_of = ops.permute_plan(assign, E)
+        counts, offsets, token_of, slot_of, row_of, scores_perm = ops.permute_plan(assign, E, scores)
         xp = ops.gather_rows_fwd(x, token_of)
         timers.stop("router")
 
+        # The score of a routed row multiplies the expert's intermediate activation (epilogue of
+        # the gate_up GEMM) instead of its output: the down projection is linear, so
+        # (s * inter) @ W_down == s * (inter @ W_down), and the combine becomes a plain sum.
         timers.start("groupGeMM")
-        gate_up, inter = ops.grouped_gemm_gateup_act_fwd(xp, w_gate_up, offsets, opts["act"], tile_cfg=opts["tile_cfg"])
-        moe_out = ops.grouped_gemm_nn(inter, w_down, offsets, tile_cfg=opts["tile_cfg"])
+        cfg = opts["tile_cfg"]
+        gate_up, inter_s = ops.grouped_gemm_gateup_act_fwd(
+            xp, w_gate_up, offsets, opts["act"], tile_cfg=cfg, row_scale=scores_perm
+        )
+        out_s = ops.grouped_gemm_nn(inter_s, w_down, offsets, tile_cfg=cfg)
         timers.stop("groupGeMM")
 
         timers.start("moe-combine")
-        y = ops.combine_fwd(moe_out, row_of, scores)
+        y = ops.combine_fwd(out_s, row_of, None)
         timers.stop("moe-combine")
 
         ctx.opts = opts
         ctx.save_for_backward(
-            x, router_gate, w_gate_up, w_down, probs, topk_idx, scores, counts, offsets, row_of, xp, gate_up, inter, moe_out
+            x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
+            xp, gate_up, inter_s,
         )
         # scores in routed-row order, in the model dtype, as the reference returns them
-        scores_perm = scores.t().reshape(-1)[slot_of.long()].to(x.dtype)
-        ctx.mark_non_differentiable(scores_perm)
+        scores_out = scores_perm.to(x.dtype)
+        ctx.mark_non_differentiable(scores_out)
         cap = opts.get("capture")
         if cap is not None:
             cap.update(logits=logits, probs=probs, topk_idx=topk_idx, scores=scores, counts=counts, offsets=offsets,
                        token_of=token_of, slot_of=slot_of, row_of=row_of)
-        return y, scores_perm
+        return y, scores_out
 
     @staticmethod
     def backward(ctx, dy, _ds_perm):
-        (x, router_gate, w_gate_up, w_down, probs, topk_idx, scores, counts, offsets, row_of, xp, gate_up, inter,
-         moe_out) = ctx.saved_tensors
+        (x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm, xp,
+         gate_up, inter_s) = ctx.saved_tensors
         opts = ctx.opts
-        E = opts["num_experts"]
+        E, K = opts["num_experts"], opts["top_k"]
         T = x.shape[0]
+        R = T * K
         cfg = opts["tile_cfg"]
         dy = dy.contiguous()
 
-        d_out, d_scores = ops.combine_bwd(dy, moe_out, row_of, scores)
-        d_inter = ops.grouped_gemm_nt(d_out, w_down, offsets, tile_cfg=cfg)
-        d_w_down = ops.grouped_gemm_wgrad(inter, d_out, offsets, E, tile_cfg=cfg) if ctx.needs_input_grad[3] else None
-        d_gate_up = ops.gated_act_bwd(gate_up, d_inter, opts["act"])
+        # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMM's A loads
+        d_inter_s = ops.grouped_gemm_nt(dy, w_down, offsets, a_row_map=token_of, n_rows=R, tile_cfg=cfg)
+        d_w_down = None
+        if ctx.needs_input_grad[3]:
+            dyp = ops.gather_rows_fwd(dy, token_of)
+            d_w_down = ops.grouped_gemm_wgrad(inter_s, dyp, offsets, E, tile_cfg=cfg)
+            del dyp
+        # gated-activation backward, with the score multiply: also yields d_scores [T,K]
+        d_gate_up, d_scores = ops.gated_act_bwd(
+            gate_up, d_inter_s, opts["act"], row_scale=scores_perm, slot_of=slot_of, tk=(T, K)
+        )
         d_w_gate_up = ops.grouped_gemm_wgrad(xp, d_gate_up, offsets, E, tile_cfg=cfg) if ctx.needs_input_grad[2] else None
 
         d_logits = ops.router_bwd(

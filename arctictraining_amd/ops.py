@@ -72,8 +72,9 @@ def router_bwd(d_scores, probs, topk_idx, counts, out_dtype, normalize: bool, lb
     return d_logits
 
 
-def permute_plan(assign: torch.Tensor, num_experts: int):
-    """assign [T,K] i32 -> counts [E], offsets [E+1], token_of [R], slot_of [R], row_of [T,K] (all i32)."""
+def permute_plan(assign: torch.Tensor, num_experts: int, scores: Optional[torch.Tensor] = None):
+    """assign [T,K] i32 -> counts [E], offsets [E+1], token_of [R], slot_of [R], row_of [T,K] (all i32) and,
+    when scores [T,K] f32 is given, scores_perm [R] f32 (else None)."""
     lib = _lib.load()
     _chk(assign, "assign", torch.int32)
     T, K = assign.shape
@@ -83,14 +84,18 @@ def permute_plan(assign: torch.Tensor, num_experts: int):
     token_of = torch.empty(R, dtype=torch.int32, device=dev)
     slot_of = torch.empty(R, dtype=torch.int32, device=dev)
     row_of = torch.empty((T, K), dtype=torch.int32, device=dev)
+    scores_perm = None
+    if scores is not None:
+        _chk(scores, "scores", torch.float32)
+        scores_perm = torch.empty(R, dtype=torch.float32, device=dev)
     ws_bytes = lib.amoe_permute_workspace_bytes(R, E)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     rc = lib.amoe_permute_plan(
-        assign.data_ptr(), T, K, E, counts.data_ptr(), offsets.data_ptr(), token_of.data_ptr(), slot_of.data_ptr(),
-        row_of.data_ptr(), ws.data_ptr(), ws.numel(), _stream()
+        assign.data_ptr(), _ptr(scores), T, K, E, counts.data_ptr(), offsets.data_ptr(), token_of.data_ptr(),
+        slot_of.data_ptr(), row_of.data_ptr(), _ptr(scores_perm), ws.data_ptr(), ws.numel(), _stream()
     )
     _lib.check(rc, "amoe_permute_plan")
-    return counts, offsets, token_of, slot_of, row_of
+    return counts, offsets, token_of, slot_of, row_of, scores_perm
 
 
 def gather_rows_fwd(x: torch.Tensor, token_of: torch.Tensor) -> torch.Tensor:
@@ -120,16 +125,18 @@ def gather_rows_bwd(d_xp: torch.Tensor, row_of: torch.Tensor, addend: Optional[t
     return dx
 
 
-def combine_fwd(moe_out: torch.Tensor, row_of: torch.Tensor, scores: torch.Tensor) -> torch.Tensor:
+def combine_fwd(moe_out: torch.Tensor, row_of: torch.Tensor, scores: Optional[torch.Tensor]) -> torch.Tensor:
+    """y[t] = sum_k scores[t,k] * moe_out[row_of[t,k]]; scores None = unweighted."""
     lib = _lib.load()
     _chk(moe_out, "moe_out")
     _chk(row_of, "row_of", torch.int32)
-    _chk(scores, "scores", torch.float32)
+    if scores is not None:
+        _chk(scores, "scores", torch.float32)
     T, K = row_of.shape
     H = moe_out.shape[1]
     y = torch.empty((T, H), dtype=moe_out.dtype, device=moe_out.device)
     rc = lib.amoe_combine_fwd(
-        moe_out.data_ptr(), row_of.data_ptr(), scores.data_ptr(), y.data_ptr(), _dtype_code(moe_out), T, K, H, _stream()
+        moe_out.data_ptr(), row_of.data_ptr(), _ptr(scores), y.data_ptr(), _dtype_code(moe_out), T, K, H, _stream()
     )
     _lib.check(rc, "amoe_combine_fwd")
     return y
@@ -167,14 +174,18 @@ def grouped_gemm_gateup_act_fwd(
     n_rows: Optional[int] = None,
     tile_cfg: int = 0,
     want_gate_up: bool = True,
+    row_scale: Optional[torch.Tensor] = None,
 ):
-    """gate_up [R,2I], inter [R,I] from xp [R,H] (or x [T,H] with a_row_map [R]) and w [E,H,2I]."""
+    """gate_up [R,2I], inter [R,I] (times row_scale [R] when given) from xp [R,H] (or x [T,H] with
+    a_row_map [R]) and w [E,H,2I]."""
     lib = _lib.load()
     _chk(xp, "xp")
     _chk(w_gate_up, "w_gate_up", xp.dtype)
     _chk(offsets, "offsets", torch.int32)
     if a_row_map is not None:
         _chk(a_row_map, "a_row_map", torch.int32)
+    if row_scale is not None:
+        _chk(row_scale, "row_scale", torch.float32)
     E, H, I2 = w_gate_up.shape
     R = int(n_rows if n_rows is not None else (a_row_map.numel() if a_row_map is not None else xp.shape[0]))
     I = I2 // 2
@@ -182,7 +193,8 @@ def grouped_gemm_gateup_act_fwd(
     inter = torch.empty((R, I), dtype=xp.dtype, device=xp.device)
     ws = _gemm_workspace(R, E, xp.device)
     rc = lib.amoe_grouped_gemm_gateup_act_fwd(
-        xp.data_ptr(), _ptr(a_row_map), w_gate_up.data_ptr(), offsets.data_ptr(), _ptr(gate_up), inter.data_ptr(),
+        xp.data_ptr(), _ptr(a_row_map), w_gate_up.data_ptr(), offsets.data_ptr(), _ptr(row_scale), _ptr(gate_up),
+        inter.data_ptr(),
         _dtype_code(xp), R, E, H, I, act, ws.data_ptr(), ws.numel(), tile_cfg, _stream()
     )
     _lib.check(rc, "amoe_grouped_gemm_gateup_act_fwd")
@@ -242,14 +254,31 @@ def grouped_gemm_wgrad(A, B, offsets, num_experts: int, tile_cfg: int = 0) -> to
     return C
 
 
-def gated_act_bwd(gate_up: torch.Tensor, d_inter: torch.Tensor, act: int = ACT_SILU) -> torch.Tensor:
+def gated_act_bwd(
+    gate_up: torch.Tensor,
+    d_inter: torch.Tensor,
+    act: int = ACT_SILU,
+    row_scale: Optional[torch.Tensor] = None,
+    slot_of: Optional[torch.Tensor] = None,
+    tk: Optional[Tuple[int, int]] = None,
+):
+    """d_gate_up [R,2I]; with row_scale [R], slot_of [R] and tk=(T,K) also d_row_scale [T,K] f32."""
     lib = _lib.load()
     _chk(gate_up, "gate_up")
     _chk(d_inter, "d_inter", gate_up.dtype)
     R, I = d_inter.shape
     d_gu = torch.empty_like(gate_up)
+    d_scale = None
+    T = K = 0
+    if row_scale is not None:
+        _chk(row_scale, "row_scale", torch.float32)
+    if slot_of is not None:
+        _chk(slot_of, "slot_of", torch.int32)
+        T, K = tk
+        d_scale = torch.empty((T, K), dtype=torch.float32, device=gate_up.device)
     rc = lib.amoe_gated_act_bwd(
-        gate_up.data_ptr(), d_inter.data_ptr(), d_gu.data_ptr(), _dtype_code(gate_up), R, I, act, _stream()
+        gate_up.data_ptr(), d_inter.data_ptr(), _ptr(row_scale), _ptr(slot_of), d_gu.data_ptr(), _ptr(d_scale),
+        _dtype_code(gate_up), R, I, T, K, act, _stream()
     )
     _lib.check(rc, "amoe_gated_act_bwd")
-    return d_gu
+    return d_gu if slot_of is None else (d_gu, d_scale)

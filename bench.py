@@ -156,6 +156,8 @@ def main():
     d_out, _ = ops.combine_bwd(dyg, out, row_of, scores)
     d_inter = ops.grouped_gemm_nt(d_out, layer.expert_down.detach(), offsets, tile_cfg=args.tile_cfg)
     d_gu = ops.gated_act_bwd(gu, d_inter)
+    slot_of, R_tk = cap["slot_of"], (T, K)
+    s_perm = scores.t().reshape(-1)[slot_of.long()].contiguous()
     d_xp = ops.grouped_gemm_nt(d_gu, layer.expert_gate_up.detach(), offsets, tile_cfg=args.tile_cfg)
     wgu_d, wd_d = layer.expert_gate_up.detach(), layer.expert_down.detach()
     es = 2 if dtype == torch.bfloat16 else 4
@@ -179,7 +181,8 @@ def main():
          (R * H + E * H * 2 * I + 3 * R * I) * es),
         ("gemm_down_fwd", lambda: ops.grouped_gemm_nn(inter, wd_d, offsets, tile_cfg=c), 2.0 * R * H * I,
          (R * I + E * I * H + R * H) * es),
-        ("gemm_dgrad_down", lambda: ops.grouped_gemm_nt(d_out, wd_d, offsets, tile_cfg=c), 2.0 * R * H * I,
+        ("gemm_dgrad_down", lambda: ops.grouped_gemm_nt(dyg, wd_d, offsets, a_row_map=token_of, n_rows=R, tile_cfg=c),
+         2.0 * R * H * I,
          (R * H + E * I * H + R * I) * es),
         ("gemm_wgrad_down", lambda: ops.grouped_gemm_wgrad(inter, d_out, offsets, E, tile_cfg=c), 2.0 * R * H * I,
          (R * I + R * H + E * I * H) * es),
@@ -188,12 +191,12 @@ def main():
         ("gemm_wgrad_gateup", lambda: ops.grouped_gemm_wgrad(xp, d_gu, offsets, E, tile_cfg=c), 4.0 * R * H * I,
          (R * H + 2 * R * I + E * H * 2 * I) * es),
         ("gather_rows_fwd", lambda: ops.gather_rows_fwd(xd, token_of), 0.0, (T + R) * H * es),
-        ("combine_fwd", lambda: ops.combine_fwd(out, row_of, scores), 0.0, (R + T) * H * es + R * 4),
-        ("combine_bwd", lambda: ops.combine_bwd(dyg, out, row_of, scores), 0.0, (T + 2 * R) * H * es + R * 8),
-        ("gated_act_bwd", lambda: ops.gated_act_bwd(gu, d_inter), 0.0, 5 * R * I * es),
+        ("combine_fwd", lambda: ops.combine_fwd(out, row_of, None), 0.0, (R + T) * H * es + R * 4),
+        ("gated_act_bwd", lambda: ops.gated_act_bwd(gu, d_inter, row_scale=s_perm, slot_of=slot_of, tk=R_tk), 0.0,
+         5 * R * I * es + 12 * R),
         ("gather_rows_bwd", lambda: ops.gather_rows_bwd(d_xp, row_of, None), 0.0, (R + T) * H * es),
         ("router_topk_fwd", lambda: ops.router_topk_fwd(cap["logits"], K, True), 0.0, T * E * (es + 4) + T * K * 8),
-        ("permute_plan", lambda: ops.permute_plan(cap["topk_idx"], E), 0.0, R * 4 * 5),
+        ("permute_plan", lambda: ops.permute_plan(cap["topk_idx"], E, scores), 0.0, R * 4 * 7),
     ]
     breakdown = []
     for name, fn, flops, nbytes in kernels:

@@ -80,12 +80,14 @@ int amoe_router_bwd(const float* d_scores, const float* probs, const int32_t* to
  *   counts [E], offsets [E+1] (exclusive prefix), token_of [R] (row -> token, the
  *   reference's token_mapped_slots), slot_of [R] (row -> flat slot f = k*T+t, the
  *   reference's pre-modulo permutation), row_of [T,K] (slot -> row, the custom path's
- *   mapped_slots).  workspace: amoe_permute_workspace_bytes(T*K, E) bytes.
+ *   mapped_slots).  Optionally scores [T,K] f32 -> scores_perm [R] f32, the scores in row
+ *   order (moe.py:379); both may be null.
+ *   workspace: amoe_permute_workspace_bytes(T*K, E) bytes.
  */
 size_t amoe_permute_workspace_bytes(int R, int E);
-int amoe_permute_plan(const int32_t* assign, int T, int K, int E, int32_t* counts, int32_t* offsets,
-                      int32_t* token_of, int32_t* slot_of, int32_t* row_of, void* workspace, size_t workspace_bytes,
-                      void* stream);
+int amoe_permute_plan(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                      int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of, float* scores_perm,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Row gather  xp[r,:] = x[token_of[r],:]  (moe.py:356; forward half of moe_scatter,
@@ -102,7 +104,8 @@ int amoe_gather_rows_bwd(const void* d_xp, const int32_t* row_of, const void* ad
 
 /*
  * Weighted combine  y[t,:] = sum_k scores[t,k] * moe_out[row_of[t,k],:]  (moe.py:450-461;
- * moe_gather, moe_gather.cpp:28-60), f32 accumulate, one rounding.
+ * moe_gather, moe_gather.cpp:28-60), f32 accumulate, one rounding.  scores == null sums the
+ * rows unweighted (for rows that were already scaled by their score upstream).
  */
 int amoe_combine_fwd(const void* moe_out, const int32_t* row_of, const float* scores, void* y, int dtype, int T,
                      int K, int H, void* stream);
@@ -121,17 +124,20 @@ size_t amoe_grouped_gemm_workspace_bytes(int R, int E);
 
 /*
  * Grouped gate_up GEMM with the gated activation fused (moe.py:54-60 + 187-191):
- *   gate_up[rows_e, :] = xp[rows_e, :] @ w_gate_up[e]          [R,2I]
- *   inter[r, i] = gate_up[r, 2i+1] * act(gate_up[r, 2i])        [R,I]
+ *   gate_up[rows_e, :] = xp[rows_e, :] @ w_gate_up[e]                          [R,2I]
+ *   inter[r, i] = row_scale[r] * gate_up[r, 2i+1] * act(gate_up[r, 2i])        [R,I]
  * xp [R,H]; w_gate_up [E,H,2I] (gate in even, up in odd columns); offsets [E+1].
  * When `a_row_map` is non-null, row r of the A operand is read from xp[a_row_map[r], :]
  * (the gather of moe.py:356 folded into the GEMM; xp is then the un-permuted [T,H]).
- * gate_up may be null when only inter is wanted.  tile_cfg: 0 = library default.
+ * row_scale [R] f32 may be null (= 1); passing the row-ordered scores folds the multiply of
+ * moe.py:460 into this epilogue (the down projection is linear, so scaling its input rows
+ * equals scaling its output rows).  gate_up may be null when only inter is wanted.
+ * tile_cfg: 0 = library default.
  */
 int amoe_grouped_gemm_gateup_act_fwd(const void* xp, const int32_t* a_row_map, const void* w_gate_up,
-                                     const int32_t* offsets, void* gate_up, void* inter, int dtype, int R, int E,
-                                     int H, int I, int act, void* workspace, size_t workspace_bytes, int tile_cfg,
-                                     void* stream);
+                                     const int32_t* offsets, const float* row_scale, void* gate_up, void* inter,
+                                     int dtype, int R, int E, int H, int I, int act, void* workspace,
+                                     size_t workspace_bytes, int tile_cfg, void* stream);
 
 /*
  * Grouped GEMM, B not transposed (moe.py:54-60):  C[rows_e,:] = A[rows_e,:] @ B[e]
@@ -158,11 +164,16 @@ int amoe_grouped_gemm_wgrad(const void* A, const void* B, const int32_t* offsets
                             int Kd, int N, int tile_cfg, void* stream);
 
 /*
- * Backward of the gated activation (autograd of moe.py:189-191):
- *   d_gate_up[r,2i]   = d_inter[r,i] * up * act'(gate)
- *   d_gate_up[r,2i+1] = d_inter[r,i] * act(gate)
+ * Backward of inter[r,i] = row_scale[r] * up * act(gate) (autograd of moe.py:189-191, and of
+ * the score multiply of moe.py:460 when row_scale carries the scores):
+ *   d_gate_up[r,2i]   = row_scale[r] * d_inter[r,i] * up * act'(gate)
+ *   d_gate_up[r,2i+1] = row_scale[r] * d_inter[r,i] * act(gate)
+ *   d_row_scale[t,k]  = sum_i d_inter[r,i] * up * act(gate)   for the slot (t,k) of row r
+ * row_scale may be null (= 1).  d_row_scale [T,K] f32 may be null; when given, slot_of [R]
+ * (row -> flat slot k*T+t) locates the slot and T*K must equal R.
  */
-int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, void* d_gate_up, int dtype, int R, int I, int act,
+int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, const float* row_scale, const int32_t* slot_of,
+                       void* d_gate_up, float* d_row_scale, int dtype, int R, int I, int T, int K, int act,
                        void* stream);
 
 #ifdef __cplusplus

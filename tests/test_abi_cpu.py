@@ -66,11 +66,12 @@ def test_router_argument_errors(lib):
 
 
 def test_permute_argument_errors(lib):
-    assert lib.amoe_permute_plan(P, 4, 2, 8, P, P, P, P, P, None, 0, None) == -1
-    assert lib.amoe_permute_plan(P, 4, 2, 8, P, P, P, P, P, P, 0, None) == -3  # workspace too small
+    assert lib.amoe_permute_plan(P, None, 4, 2, 8, P, P, P, P, P, None, None, 0, None) == -1
+    assert lib.amoe_permute_plan(P, None, 4, 2, 8, P, P, P, P, P, P, P, 0, None) == -1  # scores_perm without scores
+    assert lib.amoe_permute_plan(P, None, 4, 2, 8, P, P, P, P, P, None, P, 0, None) == -3  # workspace too small
     assert b"workspace" in lib.amoe_last_error()
-    assert lib.amoe_permute_plan(P, 1 << 20, 4096, 8, P, P, P, P, P, P, 1 << 30, None) == -2  # R >= 2^31
-    assert lib.amoe_permute_plan(P, 4, 2, 600, P, P, P, P, P, P, 1 << 20, None) == -2
+    assert lib.amoe_permute_plan(P, None, 1 << 20, 4096, 8, P, P, P, P, P, None, P, 1 << 30, None) == -2  # R >= 2^31
+    assert lib.amoe_permute_plan(P, None, 4, 2, 600, P, P, P, P, P, None, P, 1 << 20, None) == -2
 
 
 def test_row_kernel_argument_errors(lib):
@@ -80,7 +81,9 @@ def test_row_kernel_argument_errors(lib):
     assert lib.amoe_combine_fwd(P, P, P, P, 1, 4, 17, 64, None) == -2  # K > 16
     assert lib.amoe_combine_bwd(P, P, P, P, None, None, 1, 4, 2, 64, None) == -1  # d_scores is required
     assert lib.amoe_gather_rows_bwd(P, P, None, P, 1, 0, 2, 64, None) == -1
-    assert lib.amoe_gated_act_bwd(P, P, P, 1, 4, 64, 9, None) == -1  # bad activation
+    assert lib.amoe_gated_act_bwd(P, P, None, None, P, None, 1, 4, 64, 0, 0, 9, None) == -1  # bad activation
+    assert lib.amoe_gated_act_bwd(P, P, P, None, P, P, 1, 4, 64, 2, 2, 0, None) == -1  # d_row_scale needs slot_of
+    assert lib.amoe_gated_act_bwd(P, P, P, P, P, P, 1, 4, 64, 3, 2, 0, None) == -1  # T*K != R
 
 
 def test_gemm_argument_errors(lib):
@@ -94,8 +97,8 @@ def test_gemm_argument_errors(lib):
     assert lib.amoe_grouped_gemm_nn(P, None, None, P, P, 1, 128, 4, 64, 64, P, big, 0, None) == -1
     assert lib.amoe_grouped_gemm_wgrad(P, P, P, P, 1, 128, 4, 60, 64, 0, None) == -2
     assert lib.amoe_grouped_gemm_wgrad(P, P, P, P, 0, 128, 1000, 64, 64, 0, None) == -2  # E too large
-    assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, P, P, 1, 128, 4, 64, 64, 7, P, big, 0, None) == -1
-    assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, None, P, 0, 128, 4, 64, 64, 0, P, big, 0, None) == -2
+    assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, None, P, P, 1, 128, 4, 64, 64, 7, P, big, 0, None) == -1
+    assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, None, None, P, 0, 128, 4, 64, 64, 0, P, big, 0, None) == -2
 
 
 def test_missing_library_fails_loudly(monkeypatch):

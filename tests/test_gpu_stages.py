@@ -102,9 +102,13 @@ def test_router_bwd(ops, gpu_device, dtype, E, K, normalize):
 # ------------------------------------------------------------------ permutation
 def _check_plan(ops, dev, assign, E):
     T, K = assign.shape
-    counts, offsets, token_of, slot_of, row_of = ops.permute_plan(assign.to(torch.int32).to(dev), E)
+    g = torch.Generator().manual_seed(T * 7 + K)
+    s_tk = torch.rand(T, K, generator=g)
+    counts, offsets, token_of, slot_of, row_of, s_perm = ops.permute_plan(assign.to(torch.int32).to(dev), E, s_tk.to(dev))
     torch.cuda.synchronize()
     perm, tok, cnt = O.permutation(assign.long(), E)
+    assert torch.equal(s_perm.cpu(), s_tk.t().reshape(-1)[perm]), "scores in row order (moe.py:379)"
+    assert ops.permute_plan(assign.to(torch.int32).to(dev), E)[5] is None
     assert torch.equal(counts.cpu().long(), cnt), "counts"
     assert torch.equal(offsets.cpu().long(), torch.cat([torch.zeros(1, dtype=torch.int64), cnt.cumsum(0)])), "offsets"
     assert torch.equal(slot_of.cpu().long(), perm), "permutation order"
@@ -125,7 +129,7 @@ def test_permute_plan_random(ops, gpu_device, T, K, E):
 
 def test_permute_plan_worked_example(ops, gpu_device):
     assign = torch.tensor([[1, 0], [0, 1], [1, 0]])
-    counts, offsets, token_of, slot_of, row_of = ops.permute_plan(assign.to(torch.int32).to(gpu_device), 2)
+    counts, offsets, token_of, slot_of, row_of, _ = ops.permute_plan(assign.to(torch.int32).to(gpu_device), 2)
     assert slot_of.tolist() == [1, 3, 5, 0, 2, 4]
     assert token_of.tolist() == [1, 0, 2, 0, 2, 1]
     assert counts.tolist() == [3, 3] and offsets.tolist() == [0, 3, 6]
@@ -185,6 +189,8 @@ def test_gather_and_combine(ops, gpu_device, dtype, T, K, H, E):
     y = ops.combine_fwd(out.to(d), row_d, s_tk.to(d))
     ref = O.combine(out.double(), tok, s_perm.double(), K)
     assert O.rel_l2(y.cpu(), ref) <= _tol(dtype)
+    y1 = ops.combine_fwd(out.to(d), row_d, None)
+    assert O.rel_l2(y1.cpu(), O.combine(out.double(), tok, torch.ones(R, dtype=torch.float64), K)) <= _tol(dtype)
 
     dy = torch.randn(T, H, generator=g).to(dtype)
     d_out, d_s = ops.combine_bwd(dy.to(d), out.to(d), row_d, s_tk.to(d))
@@ -211,6 +217,23 @@ def test_gated_act_bwd(ops, gpu_device, dtype, act):
     inter = gu64[:, 1::2] * O.activation(act)(gu64[:, 0::2])
     inter.backward(di.double())
     assert O.rel_l2(got.cpu(), gu64.grad) <= (5e-3 if dtype == torch.bfloat16 else 2e-5)
+    # with the score folded in: inter = s_r * up * act(gate); also the score gradient per slot
+    T, K = 25, 4
+    assign = torch.stack([torch.randperm(8, generator=g)[:K] for _ in range(T)])
+    perm, tok, _ = O.permutation(assign, 8)
+    s_perm = torch.rand(R, generator=g) + 0.1
+    got, d_s = ops.gated_act_bwd(
+        gu.to(gpu_device), di.to(gpu_device), code, row_scale=s_perm.to(gpu_device),
+        slot_of=perm.to(torch.int32).to(gpu_device), tk=(T, K),
+    )
+    gu64 = gu.double().requires_grad_(True)
+    s64 = s_perm.double().requires_grad_(True)
+    inter = s64[:, None] * gu64[:, 1::2] * O.activation(act)(gu64[:, 0::2])
+    inter.backward(di.double())
+    assert O.rel_l2(got.cpu(), gu64.grad) <= (5e-3 if dtype == torch.bfloat16 else 2e-5)
+    ref_ds = torch.zeros(R, dtype=torch.float64)
+    ref_ds[perm] = s64.grad
+    assert O.rel_l2(d_s.cpu(), ref_ds.view(K, T).t()) <= 2e-5
 
 
 # ------------------------------------------------------------------ grouped GEMMs
@@ -332,6 +355,13 @@ def test_gateup_activation_fused(ops, gpu_device, dtype, cfg, act):
             xp.to(gpu_device), w.to(gpu_device), offs, code, tile_cfg=cfg, want_gate_up=False
         )
         assert torch.equal(inter2, inter)
+    # row scale folded into the epilogue
+    rs = torch.rand(R, generator=g) + 0.25
+    gu3, inter3 = ops.grouped_gemm_gateup_act_fwd(
+        xp.to(gpu_device), w.to(gpu_device), offs, code, tile_cfg=cfg, row_scale=rs.to(gpu_device)
+    )
+    assert torch.equal(gu3, gu)
+    assert O.rel_l2(inter3.cpu(), ref_inter * rs.double()[:, None]) <= (BF16_TOL if dtype == torch.bfloat16 else 2e-5)
 
 
 def test_grouped_gemm_rows_outside_groups_untouched(ops, gpu_device):
