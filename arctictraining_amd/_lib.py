@@ -55,7 +55,8 @@ SIGNATURES = {
     ),
     "amoe_grouped_gemm_wgrad": (
         _c_int,
-        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_void_p],
     ),
     "amoe_gated_act_bwd": (
         _c_int,

@@ -25,13 +25,13 @@ int amoe_bf16_nn(const void* A, const int32_t* a_row_map, const void* B, const i
                  int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s);
 int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                  int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s);
-int amoe_bf16_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int R, int E, int Kd, int N,
-                    int tile_cfg, hipStream_t s);
+int amoe_bf16_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
+                    const int32_t* offsets, void* C, int R, int E, int Kd, int N, int tile_cfg, hipStream_t s);
 int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                   int Kred, int N, int ldb, long long strideB, bool b_kc, void* workspace, size_t workspace_bytes,
                   hipStream_t s);
-int amoe_f32_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int R, int E, int Kd, int N,
-                   hipStream_t s);
+int amoe_f32_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
+                   const int32_t* offsets, void* C, int R, int E, int Kd, int N, hipStream_t s);
 int amoe_launch_gated_act_fwd(const void* gu, const float* row_scale, void* inter, int dtype, int R, int I, int act,
                               hipStream_t s);
 
@@ -44,7 +44,7 @@ int check_gemm_common(const char* what, int dtype, int R, int E, int d0, int d1,
     AMOE_REQUIRE(R > 0 && E > 0 && d0 > 0 && d1 > 0, AMOE_ERR_BAD_ARG, "%s: sizes must be positive (R=%d E=%d %d %d)",
                  what, R, E, d0, d1);
     AMOE_REQUIRE(E <= AMOE_MAX_EXPERTS, AMOE_ERR_UNSUPPORTED, "%s: E=%d exceeds %d", what, E, AMOE_MAX_EXPERTS);
-    AMOE_REQUIRE(tile_cfg >= 0 && tile_cfg <= 5, AMOE_ERR_BAD_ARG, "%s: tile_cfg %d outside 0..5", what, tile_cfg);
+    AMOE_REQUIRE(tile_cfg >= 0 && tile_cfg <= 5 && tile_cfg != 4, AMOE_ERR_BAD_ARG, "%s: tile_cfg %d is not one of 0, 1, 2, 3, 5", what, tile_cfg);
     AMOE_REQUIRE((long long)R * d0 < (1ll << 32) && (long long)R * d1 < (1ll << 32) && (long long)d0 * d1 < (1ll << 32),
                  AMOE_ERR_UNSUPPORTED, "%s: an operand exceeds 2^32 elements", what);
     return AMOE_OK;
@@ -133,17 +133,19 @@ AMOE_EXPORT int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, co
                          workspace, workspace_bytes, s);
 }
 
-AMOE_EXPORT int amoe_grouped_gemm_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int dtype, int R,
+AMOE_EXPORT int amoe_grouped_gemm_wgrad(const void* A, const int32_t* a_row_map, const void* B,
+                                        const int32_t* b_row_map, const int32_t* offsets, void* C, int dtype, int R,
                                         int E, int Kd, int N, int tile_cfg, void* stream)
 {
     const char* what = "grouped_gemm_wgrad";
     AMOE_REQUIRE(A && B && offsets && C, AMOE_ERR_BAD_ARG, "%s: null pointer", what);
+    AMOE_REQUIRE(!(a_row_map && b_row_map), AMOE_ERR_UNSUPPORTED, "%s: at most one operand may be gathered", what);
     int rc = check_gemm_common(what, dtype, R, E, Kd, N, tile_cfg);
     if (rc) return rc;
     const int vec = dtype == AMOE_BF16 ? 8 : 4;
     AMOE_REQUIRE(Kd % vec == 0 && N % vec == 0, AMOE_ERR_UNSUPPORTED, "%s: extents (%d, %d) must be multiples of %d",
                  what, Kd, N, vec);
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == AMOE_BF16) return amoe_bf16_wgrad(A, B, offsets, C, R, E, Kd, N, tile_cfg, s);
-    return amoe_f32_wgrad(A, B, offsets, C, R, E, Kd, N, s);
+    if (dtype == AMOE_BF16) return amoe_bf16_wgrad(A, a_row_map, B, b_row_map, offsets, C, R, E, Kd, N, tile_cfg, s);
+    return amoe_f32_wgrad(A, a_row_map, B, b_row_map, offsets, C, R, E, Kd, N, s);
 }

@@ -42,6 +42,7 @@ struct GemmArgs {
     bf16_t* C;
     bf16_t* C2;
     const int32_t* a_row_map;
+    const int32_t* b_row_map;  // weight gradient only
     const float* row_scale;  // gated epilogue: inter[r,:] is multiplied by row_scale[r] (null = 1)
     const int32_t* offsets;
     const int4* tile_map;
@@ -54,6 +55,7 @@ struct GemmArgs {
     int N;        // output columns
     int n_ntiles;
     int n_mt;     // wgrad mode: M tiles per expert
+    int rows_total;  // weight gradient: length of the row maps
     int gm, gn;   // blocks of one XCD work on super-tiles of gm x gn tiles
     int sn;       // super-tiles along N
 };
@@ -125,7 +127,8 @@ __device__ __forceinline__ void lds_barrier()
 using T_ = std::true_type;
 using F_ = std::false_type;
 
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT>
+// MAPS (weight gradient only): 1 = the rows of A, 2 = the rows of B are gathered through a row map
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
 __global__ void __launch_bounds__(WGM * WGN * 64)
 grouped_gemm_bf16_kernel(GemmArgs p)
 {
@@ -133,6 +136,8 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr bool WGRAD = !A_KC;
+    constexpr bool A_MAP = WGRAD && (MAPS & 1), B_MAP = WGRAD && (MAPS & 2);
+    static_assert(WGRAD || MAPS == 0, "row-grouped launches gather through the per-thread row plan");
     static_assert(TN % 2 == 0, "N tiles come in even/odd pairs");
     static_assert(!WGRAD || (TM % 2 == 0 && !B_KC), "wgrad pairs both operands");
     static_assert(BM >= 128 && BN >= 128, "K-strided swizzle needs 16 chunks per row");
@@ -205,7 +210,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             constexpr int CPR = BM / 8;
             const int krow = c / CPR, mc = (c % CPR) ^ (((krow >> 3) & 1) << 3);
             const int col = min(m0 + mc * 8, p.M - 8);
-            aoff[i] = (uint32_t)krow * (uint32_t)p.lda + col;
+            aoff[i] = A_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.lda + col;
             a_kr[i] = krow;
         }
     }
@@ -224,43 +229,75 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             constexpr int CPR = BN / 8;
             const int krow = c / CPR, nc = (c % CPR) ^ (((krow >> 3) & 1) << 3);
             const int col = min(n0 + nc * 8, p.N - 8);
-            boff[i] = (uint32_t)krow * (uint32_t)p.ldb + col;
+            boff[i] = B_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.ldb + col;
             b_kr[i] = krow;
         }
     }
     if (!WGRAD) {
         Bb += (long long)e * p.strideB;
     } else {
-        Ab += (long long)r0 * p.lda;
-        Bb += (long long)r0 * p.ldb;
+        if (!A_MAP) Ab += (long long)r0 * p.lda;
+        if (!B_MAP) Bb += (long long)r0 * p.ldb;
     }
     const int k_rows = r1 - r0;  // wgrad: rows of this expert
 
+    // Gathered operands of the weight gradient: the source row of a chunk changes with every K
+    // tile, so it is looked up one tile ahead (a_nxt / b_nxt, fetched right before the loads of
+    // the previous tile are issued) and moved to a_use / b_use when its own loads go out.
+    int a_use[PER_A], a_nxt[PER_A], b_use[PER_B], b_nxt[PER_B];
+    auto fetch_a_idx = [&](int kt, int (&dst)[PER_A]) {
+#pragma unroll
+        for (int i = 0; i < PER_A; ++i) dst[i] = p.a_row_map[min(r0 + kt * BK + a_kr[i], p.rows_total - 1)];
+    };
+    auto fetch_b_idx = [&](int kt, int (&dst)[PER_B]) {
+#pragma unroll
+        for (int i = 0; i < PER_B; ++i) dst[i] = p.b_row_map[min(r0 + kt * BK + b_kr[i], p.rows_total - 1)];
+    };
+
     // wgrad: rows past the end of the expert read a block of zeros instead (only the last K
     // tile of an expert can be ragged, the select costs two VALU ops per load)
-    auto issue_a = [&](int kt, auto LO, auto HI) {
+    auto dma_a = [&](int kt, auto LO, auto HI, const int (&idx)[PER_A]) {
         constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
         const int k0 = kt * BK;
         u32x4_t* sa = smem + (kt & (NSTAGE - 1)) * STAGE + wave * 64;
-        const bf16_t* a_base = A_KC ? Ab + k0 : Ab + (long long)k0 * p.lda;
+        const bf16_t* a_base = A_KC ? Ab + k0 : (A_MAP ? Ab : Ab + (long long)k0 * p.lda);
 #pragma unroll
         for (int i = lo; i < hi; ++i) {
             const bf16_t* src = a_base + aoff[i];
+            if (A_MAP) src += (long long)idx[i] * p.lda;
             if (WGRAD) src = (k0 + a_kr[i] < k_rows) ? src : reinterpret_cast<const bf16_t*>(g_zero_chunk);
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sa + NT * i), 16, 0, 0);
         }
     };
-    auto issue_b = [&](int kt, auto LO, auto HI) {
+    auto dma_b = [&](int kt, auto LO, auto HI, const int (&idx)[PER_B]) {
         constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
         const int k0 = kt * BK;
         u32x4_t* sb = smem + (kt & (NSTAGE - 1)) * STAGE + A_CH + wave * 64;
-        const bf16_t* b_base = B_KC ? Bb + k0 : Bb + (long long)k0 * p.ldb;
+        const bf16_t* b_base = B_KC ? Bb + k0 : (B_MAP ? Bb : Bb + (long long)k0 * p.ldb);
 #pragma unroll
         for (int i = lo; i < hi; ++i) {
             const bf16_t* src = b_base + boff[i];
+            if (B_MAP) src += (long long)idx[i] * p.ldb;
             if (WGRAD) src = (k0 + b_kr[i] < k_rows) ? src : reinterpret_cast<const bf16_t*>(g_zero_chunk);
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sb + NT * i), 16, 0, 0);
         }
+    };
+    // steady-state issue: rotate the looked-up rows when the first half of a tile goes out
+    auto issue_a = [&](int kt, auto LO, auto HI) {
+        if (A_MAP && decltype(LO)::value == 0) {
+#pragma unroll
+            for (int i = 0; i < PER_A; ++i) a_use[i] = a_nxt[i];
+            fetch_a_idx(kt + 1, a_nxt);
+        }
+        dma_a(kt, LO, HI, a_use);
+    };
+    auto issue_b = [&](int kt, auto LO, auto HI) {
+        if (B_MAP && decltype(LO)::value == 0) {
+#pragma unroll
+            for (int i = 0; i < PER_B; ++i) b_use[i] = b_nxt[i];
+            fetch_b_idx(kt + 1, b_nxt);
+        }
+        dma_b(kt, LO, HI, b_use);
     };
 
     mfma_f32x16 acc[TM][TN];
@@ -387,15 +424,29 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     mfma_bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
 
     // prologue: tiles 0..2 and the A half of tile 3 go out, tile 0 is awaited
+    {
+        // row lookups of the first four tiles go out together, ahead of their loads
+        int ia[NSTAGE][PER_A], ib[NSTAGE][PER_B];
 #pragma unroll
-    for (int t = 0; t < NSTAGE - 1; ++t) {
-        if (t < kt_count) {
-            issue_a(t, IC0{}, A_ALL{});
-            issue_b(t, IC0{}, B_ALL{});
+        for (int t = 0; t < NSTAGE; ++t) {
+            if (A_MAP) fetch_a_idx(t, ia[t]);
+            if (B_MAP) fetch_b_idx(t, ib[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < NSTAGE - 1; ++t) {
+            if (t < kt_count) {
+                dma_a(t, IC0{}, A_ALL{}, ia[t]);
+                dma_b(t, IC0{}, B_ALL{}, ib[t]);
+            }
+        }
+        if (kt_count > NSTAGE - 1) dma_a(NSTAGE - 1, IC0{}, A_ALL{}, ia[NSTAGE - 1]);
+        if (A_MAP) fetch_a_idx(NSTAGE, a_nxt);          // next A tile to go out is tile 4
+        if (B_MAP) {
+#pragma unroll
+            for (int i = 0; i < PER_B; ++i) b_nxt[i] = ib[NSTAGE - 1][i];  // next B tile is tile 3
         }
     }
     if (kt_count > NSTAGE - 1) {
-        issue_a(NSTAGE - 1, IC0{}, A_ALL{});
         lds_barrier<2 * PER + PER_A>();
     } else {
         lds_barrier<0>();
@@ -509,10 +560,10 @@ grouped_gemm_bf16_kernel(GemmArgs p)
 }
 
 // ------------------------------------------------------------------ host side
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT>
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
 int launch_cfg(const GemmArgs& a, int grid, hipStream_t s)
 {
-    auto kern = grouped_gemm_bf16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT>;
+    auto kern = grouped_gemm_bf16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS>;
     constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool attr_done = false;
     if (!attr_done) {
@@ -538,22 +589,20 @@ inline TileCfg pick_cfg(int tile_cfg)
         case 1: return {128, 128};
         case 2: return {256, 128};
         case 3: return {256, 256};
-        case 4: return {256, 256};
         case 5: return {256, 256};
         default: return {256, 256};
     }
 }
 
-template <bool A_KC, bool B_KC, int EPI, int ACT>
+template <bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
 int launch_any(const GemmArgs& a, int tile_cfg, int grid, hipStream_t s)
 {
     switch (tile_cfg) {
-        case 1: return launch_cfg<128, 128, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
-        case 3: return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
-        case 4: return launch_cfg<256, 256, 2, 4, A_KC, B_KC, EPI, ACT>(a, grid, s);
-        case 5: return launch_cfg<256, 256, 4, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
-        case 2: return launch_cfg<256, 128, 2, 2, A_KC, B_KC, EPI, ACT>(a, grid, s);
-        default: return launch_cfg<256, 256, 2, 4, A_KC, B_KC, EPI, ACT>(a, grid, s);  // 8 waves, 128x64 per wave
+        case 1: return launch_cfg<128, 128, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+        case 3: return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+        case 5: return launch_cfg<256, 256, 4, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+        case 2: return launch_cfg<256, 128, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+        default: return launch_cfg<256, 256, 2, 4, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);  // 8 waves, 128x64 per wave
     }
 }
 
@@ -657,14 +706,17 @@ int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const i
                                              /*ldb=*/N, (long long)Kd * N, workspace, workspace_bytes, tile_cfg, s);
 }
 
-int amoe_bf16_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int R, int E, int Kd, int N,
-                    int tile_cfg, hipStream_t s)
+int amoe_bf16_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
+                    const int32_t* offsets, void* C, int R, int E, int Kd, int N, int tile_cfg, hipStream_t s)
 {
     TileCfg tc = pick_cfg(tile_cfg);
     GemmArgs a = {};
     a.A = (const bf16_t*)A;
     a.B = (const bf16_t*)B;
     a.C = (bf16_t*)C;
+    a.a_row_map = a_row_map;
+    a.b_row_map = b_row_map;
+    a.rows_total = R;
     a.offsets = offsets;
     a.lda = Kd;
     a.ldb = N;
@@ -678,5 +730,7 @@ int amoe_bf16_wgrad(const void* A, const void* B, const int32_t* offsets, void* 
     long long grid = 0;
     int rc = set_supertiles(a, (long long)E * a.n_mt, &grid);
     if (rc) return rc;
+    if (a_row_map) return launch_any<false, false, EPI_STORE, 0, 1>(a, tile_cfg, (int)grid, s);
+    if (b_row_map) return launch_any<false, false, EPI_STORE, 0, 2>(a, tile_cfg, (int)grid, s);
     return launch_any<false, false, EPI_STORE, 0>(a, tile_cfg, (int)grid, s);
 }

@@ -19,6 +19,7 @@ struct GemmArgsF32 {
     const float* B;
     float* C;
     const int32_t* a_row_map;
+    const int32_t* b_row_map;  // weight gradient only
     const int32_t* offsets;
     const int4* tile_map;
     const int32_t* n_mtiles;
@@ -64,6 +65,7 @@ grouped_gemm_f32_kernel(GemmArgsF32 p)
 
     // per-thread source coordinates
     long long a_src;
+    int a_col = 0, b_col = 0;  // column offsets of the gathered weight-gradient operands
     int a_k;  // k offset inside the tile
     if (A_KC) {
         const int m = tid >> 2;
@@ -74,7 +76,8 @@ grouped_gemm_f32_kernel(GemmArgsF32 p)
     } else {
         a_k = tid >> 4;
         const int m4 = (tid & 15) * 4;
-        a_src = (long long)a_k * p.lda + min(m0 + m4, p.M - 4);
+        a_col = min(m0 + m4, p.M - 4);
+        a_src = (long long)a_k * p.lda + a_col;
     }
     long long b_src;
     int b_k;
@@ -85,7 +88,8 @@ grouped_gemm_f32_kernel(GemmArgsF32 p)
     } else {
         b_k = tid >> 4;
         const int n4 = (tid & 15) * 4;
-        b_src = (long long)b_k * p.ldb + min(n0 + n4, p.N - 4);
+        b_col = min(n0 + n4, p.N - 4);
+        b_src = (long long)b_k * p.ldb + b_col;
     }
 
     mfma_f32x16 acc;
@@ -97,11 +101,19 @@ grouped_gemm_f32_kernel(GemmArgsF32 p)
         f32x4_t va, vb;
         if (A_KC) {
             va = (k0 + a_k < k_len) ? *reinterpret_cast<const f32x4_t*>(Ab + a_src + k0) : zero4;
+        } else if (p.a_row_map) {
+            va = (k0 + a_k < k_len) ? *reinterpret_cast<const f32x4_t*>(
+                                          p.A + (long long)p.a_row_map[r0 + k0 + a_k] * p.lda + a_col)
+                                    : zero4;
         } else {
             va = (k0 + a_k < k_len) ? *reinterpret_cast<const f32x4_t*>(Ab + a_src + (long long)k0 * p.lda) : zero4;
         }
         if (B_KC) {
             vb = (k0 + b_k < k_len) ? *reinterpret_cast<const f32x4_t*>(Bb + b_src + k0) : zero4;
+        } else if (WGRAD && p.b_row_map) {
+            vb = (k0 + b_k < k_len) ? *reinterpret_cast<const f32x4_t*>(
+                                          p.B + (long long)p.b_row_map[r0 + k0 + b_k] * p.ldb + b_col)
+                                    : zero4;
         } else {
             vb = (k0 + b_k < k_len) ? *reinterpret_cast<const f32x4_t*>(Bb + b_src + (long long)k0 * p.ldb) : zero4;
         }
@@ -172,10 +184,12 @@ int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const 
     return amoe_check_launch("grouped_gemm_f32");
 }
 
-int amoe_f32_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int R, int E, int Kd, int N,
-                   hipStream_t s)
+int amoe_f32_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
+                   const int32_t* offsets, void* C, int R, int E, int Kd, int N, hipStream_t s)
 {
     GemmArgsF32 a = {};
+    a.a_row_map = a_row_map;
+    a.b_row_map = b_row_map;
     a.A = (const float*)A;
     a.B = (const float*)B;
     a.C = (float*)C;

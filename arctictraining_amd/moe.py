@@ -107,16 +107,16 @@ class _ExpertLayerFn(torch.autograd.Function):
         probs, topk_idx, scores = ops.router_topk_fwd(logits, K, opts["normalize"])
         assign = topk_idx if replay is None else replay.to(torch.int32).contiguous()
         counts, offsets, token_of, slot_of, row_of, scores_perm = ops.permute_plan(assign, E, scores)
-        xp = ops.gather_rows_fwd(x, token_of)
         timers.stop("router")
 
-        # The score of a routed row multiplies the expert's intermediate activation (epilogue of
+        # The gather x[token_of] (moe.py:356) happens inside the GEMMs' A loads: the routed copy
+        # of the activations is never written.  The score of a routed row multiplies the expert's intermediate activation (epilogue of
         # the gate_up GEMM) instead of its output: the down projection is linear, so
         # (s * inter) @ W_down == s * (inter @ W_down), and the combine becomes a plain sum.
         timers.start("groupGeMM")
         cfg = opts["tile_cfg"]
         gate_up, inter_s = ops.grouped_gemm_gateup_act_fwd(
-            xp, w_gate_up, offsets, opts["act"], tile_cfg=cfg, row_scale=scores_perm
+            x, w_gate_up, offsets, opts["act"], a_row_map=token_of, n_rows=T * K, tile_cfg=cfg, row_scale=scores_perm
         )
         out_s = ops.grouped_gemm_nn(inter_s, w_down, offsets, tile_cfg=cfg)
         timers.stop("groupGeMM")
@@ -128,7 +128,7 @@ class _ExpertLayerFn(torch.autograd.Function):
         ctx.opts = opts
         ctx.save_for_backward(
             x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
-            xp, gate_up, inter_s,
+            gate_up, inter_s,
         )
         # scores in routed-row order, in the model dtype, as the reference returns them
         scores_out = scores_perm.to(x.dtype)
@@ -141,7 +141,7 @@ class _ExpertLayerFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy, _ds_perm):
-        (x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm, xp,
+        (x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
          gate_up, inter_s) = ctx.saved_tensors
         opts = ctx.opts
         E, K = opts["num_experts"], opts["top_k"]
@@ -150,18 +150,18 @@ class _ExpertLayerFn(torch.autograd.Function):
         cfg = opts["tile_cfg"]
         dy = dy.contiguous()
 
-        # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMM's A loads
+        # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMMs' loads
         d_inter_s = ops.grouped_gemm_nt(dy, w_down, offsets, a_row_map=token_of, n_rows=R, tile_cfg=cfg)
         d_w_down = None
         if ctx.needs_input_grad[3]:
-            dyp = ops.gather_rows_fwd(dy, token_of)
-            d_w_down = ops.grouped_gemm_wgrad(inter_s, dyp, offsets, E, tile_cfg=cfg)
-            del dyp
+            d_w_down = ops.grouped_gemm_wgrad(inter_s, dy, offsets, E, tile_cfg=cfg, b_row_map=token_of)
         # gated-activation backward, with the score multiply: also yields d_scores [T,K]
         d_gate_up, d_scores = ops.gated_act_bwd(
             gate_up, d_inter_s, opts["act"], row_scale=scores_perm, slot_of=slot_of, tk=(T, K)
         )
-        d_w_gate_up = ops.grouped_gemm_wgrad(xp, d_gate_up, offsets, E, tile_cfg=cfg) if ctx.needs_input_grad[2] else None
+        d_w_gate_up = None
+        if ctx.needs_input_grad[2]:
+            d_w_gate_up = ops.grouped_gemm_wgrad(x, d_gate_up, offsets, E, tile_cfg=cfg, a_row_map=token_of)
 
         d_logits = ops.router_bwd(
             d_scores, probs, topk_idx, counts, x.dtype, opts["normalize"], opts["loss_coeff"] / T / opts["ep_size"]

@@ -237,18 +237,26 @@ def grouped_gemm_nt(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 
     return C
 
 
-def grouped_gemm_wgrad(A, B, offsets, num_experts: int, tile_cfg: int = 0) -> torch.Tensor:
-    """C[e] = A[rows_e,:]^T @ B[rows_e,:];  A [R,Kd], B [R,N] -> C [E,Kd,N]."""
+def grouped_gemm_wgrad(A, B, offsets, num_experts: int, tile_cfg: int = 0, a_row_map=None, b_row_map=None) -> torch.Tensor:
+    """C[e] = A[rows_e,:]^T @ B[rows_e,:];  A [R,Kd], B [R,N] -> C [E,Kd,N].  With a_row_map [R] (or
+    b_row_map [R]) the rows of A (or B) are gathered from a smaller matrix inside the kernel."""
     lib = _lib.load()
     _chk(A, "A")
     _chk(B, "B", A.dtype)
     _chk(offsets, "offsets", torch.int32)
-    R, Kd = A.shape
+    if a_row_map is not None:
+        _chk(a_row_map, "a_row_map", torch.int32)
+    if b_row_map is not None:
+        _chk(b_row_map, "b_row_map", torch.int32)
+    R = a_row_map.numel() if a_row_map is not None else A.shape[0]
+    if b_row_map is None and a_row_map is not None and B.shape[0] != R:
+        raise RuntimeError("B must have one row per routed row")
+    Kd = A.shape[1]
     N = B.shape[1]
     C = torch.empty((num_experts, Kd, N), dtype=A.dtype, device=A.device)
     rc = lib.amoe_grouped_gemm_wgrad(
-        A.data_ptr(), B.data_ptr(), offsets.data_ptr(), C.data_ptr(), _dtype_code(A), R, num_experts, Kd, N, tile_cfg,
-        _stream()
+        A.data_ptr(), _ptr(a_row_map), B.data_ptr(), _ptr(b_row_map), offsets.data_ptr(), C.data_ptr(), _dtype_code(A), R,
+        num_experts, Kd, N, tile_cfg, _stream()
     )
     _lib.check(rc, "amoe_grouped_gemm_wgrad")
     return C

@@ -159,9 +159,13 @@ int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, const void* B,
 /*
  * Grouped weight-gradient GEMM:  C[e] = A[rows_e,:]^T @ B[rows_e,:]   (zeros for an empty
  * expert).  A [R,Kd], B [R,N], C [E,Kd,N].  The autograd of moe.py:59 w.r.t. B[e].
+ * One of the operands may be gathered: with a_row_map [R], row r of A is read from
+ * A[a_row_map[r],:] (A then has as many rows as the map addresses); likewise b_row_map for B.
+ * tile_cfg: 0 default, or 1, 2, 3, 5 (other tile shapes, for tuning).
  */
-int amoe_grouped_gemm_wgrad(const void* A, const void* B, const int32_t* offsets, void* C, int dtype, int R, int E,
-                            int Kd, int N, int tile_cfg, void* stream);
+int amoe_grouped_gemm_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
+                            const int32_t* offsets, void* C, int dtype, int R, int E, int Kd, int N, int tile_cfg,
+                            void* stream);
 
 /*
  * Backward of inter[r,i] = row_scale[r] * up * act(gate) (autograd of moe.py:189-191, and of

@@ -268,9 +268,8 @@ GEMM_CASES = [
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 1),
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 2),
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 3),
-    (torch.bfloat16, 1000, 8, 128, 192, "ragged", 4),
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 5),
-    (torch.bfloat16, 3000, 5, 320, 576, "ragged", 4),
+    (torch.bfloat16, 3000, 5, 320, 576, "ragged", 0),
     (torch.bfloat16, 3000, 5, 320, 576, "holes", 5),
     (torch.bfloat16, 777, 6, 256, 320, "holes", 0),
     (torch.bfloat16, 2500, 16, 512, 384, "ragged", 0),
@@ -326,10 +325,28 @@ def test_grouped_gemm_nn_nt_wgrad(ops, gpu_device, dtype, R, E, Kd, N, cname, cf
     for e in range(E):
         if int(counts[e]) == 0:
             assert bool((W[e] == 0).all()), "empty expert must produce exact zeros"
+    # weight gradient with one operand gathered through a row map inside the kernel
+    Tn = max(R // 2, 1)
+    rmap = torch.randint(0, Tn, (R,), generator=g)
+    rmap_d = rmap.to(torch.int32).to(d)
+    srcA = torch.randn(Tn, Kd, generator=g).to(dtype)
+    Wa = ops.grouped_gemm_wgrad(srcA.to(d), G.to(d), offs, E, tile_cfg=cfg, a_row_map=rmap_d)
+    srcB = torch.randn(Tn, N, generator=g).to(dtype)
+    Wb = ops.grouped_gemm_wgrad(A.to(d), srcB.to(d), offs, E, tile_cfg=cfg, b_row_map=rmap_d)
+    refA = torch.zeros(E, Kd, N, dtype=torch.float64)
+    refB = torch.zeros(E, Kd, N, dtype=torch.float64)
+    start = 0
+    for e in range(E):
+        end = int(cs[e])
+        refA[e] = srcA.double()[rmap[start:end]].t() @ G.double()[start:end]
+        refB[e] = A.double()[start:end].t() @ srcB.double()[rmap[start:end]]
+        start = end
+    assert O.rel_l2(Wa.cpu(), refA) <= tol, "wgrad + A row map"
+    assert O.rel_l2(Wb.cpu(), refB) <= tol, "wgrad + B row map"
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("cfg", [0, 1, 3, 4, 5])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 5])
 @pytest.mark.parametrize("act", ["silu", "gpt_oss"])
 def test_gateup_activation_fused(ops, gpu_device, dtype, cfg, act):
     _say("gateup", dtype, cfg, act)
