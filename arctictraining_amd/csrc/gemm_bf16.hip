@@ -12,11 +12,16 @@
 //     16 bytes; chunk kc of row r sits at position kc ^ ((r >> 2) & 3), which makes the 32
 //     rows a half-wave reads cover every group of 4 banks exactly twice and the 4 lanes of
 //     each quad distinct groups: conflict-free on the 64-bank LDS of gfx950;
-//   * eight ds_read_b32 + v_perm when it is K-strided: a dword holds two ADJACENT columns of
-//     one k row, so one set of reads feeds a PAIR of MFMA tiles, one taking the even and one
-//     the odd columns.  The pair's accumulators then hold (col 2j, col 2j+1) in the same lane
-//     and register, which makes the stores packed 4-byte and lets the gated activation
-//     (gate = even, up = odd column) run on registers in the epilogue.
+//   * two ds_read_b64_tr_b16 (the transposing LDS read of gfx950) when it is K-strided, i.e.
+//     stored [k][column] with the columns contiguous.  The 16 lanes of a group together read a
+//     4 (k) x 16 (columns) block -- lane j supplies the address of k row j/4, columns
+//     4*(j%4)..+3 -- and lane i of the group receives column i for the 4 k rows, which is the
+//     MFMA operand layout.  16-byte chunk c of k row k sits at position c ^ ((k & 3) << 2), so
+//     the four k rows a half-wave reads fall into the four different quarters of the banks.
+// Every operand layout therefore yields the same accumulator layout: lane l of a 32x32 tile
+// holds column l%32.  In the epilogue neighbouring lanes swap one value (DPP) so that each
+// lane stores a packed pair of adjacent columns of ONE row; for the gate_up GEMM that pair is
+// (gate, up) of one intermediate column, so the gated activation runs on registers.
 //
 // Row-grouped launches take their (expert, first row, end row) per M tile from a tile map
 // that a small kernel builds on the device from the expert offsets: no host sync, empty
@@ -105,11 +110,29 @@ tile_map_kernel(const int32_t* __restrict__ offsets, int E, int bm, int4* __rest
     }
 }
 
-__device__ __forceinline__ uint32_t perm_lo(uint32_t w1, uint32_t w0) { return __builtin_amdgcn_perm(w1, w0, 0x05040100u); }
-__device__ __forceinline__ uint32_t perm_hi(uint32_t w1, uint32_t w0) { return __builtin_amdgcn_perm(w1, w0, 0x07060302u); }
+typedef short tr_i16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) tr_i16x4* tr_lptr_t;
+
+// value of the lane whose index differs in bit 0 / bit 1 (DPP quad permutes, no LDS traffic)
+__device__ __forceinline__ float lane_xor1(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ float lane_xor2(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+}
 
 // 16 zero bytes that masked lanes of a direct-to-LDS load read instead of out-of-range rows
 __device__ __attribute__((aligned(16))) uint32_t g_zero_chunk[4] = {0u, 0u, 0u, 0u};
+
+// Wave-uniform load of one int32 from memory this kernel never writes: read through the
+// constant address space, which makes it a scalar load (its own counter, tracked by the
+// compiler) instead of a vector load.
+__device__ __forceinline__ int scalar_load_i32(const int32_t* ptr)
+{
+    return *(const __attribute__((address_space(4))) int32_t*)ptr;
+}
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -138,8 +161,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     constexpr bool WGRAD = !A_KC;
     constexpr bool A_MAP = WGRAD && (MAPS & 1), B_MAP = WGRAD && (MAPS & 2);
     static_assert(WGRAD || MAPS == 0, "row-grouped launches gather through the per-thread row plan");
-    static_assert(TN % 2 == 0, "N tiles come in even/odd pairs");
-    static_assert(!WGRAD || (TM % 2 == 0 && !B_KC), "wgrad pairs both operands");
+    static_assert(!WGRAD || !B_KC, "the weight gradient reduces over rows: both operands are K-strided");
     static_assert(BM >= 128 && BN >= 128, "K-strided swizzle needs 16 chunks per row");
     constexpr int A_CH = BM * 4, B_CH = BN * 4;   // 16-byte chunks per stage (a 32-wide K row is 4 chunks)
     constexpr int STAGE = A_CH + B_CH;
@@ -197,6 +219,12 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     int a_kr[PER_A], b_kr[PER_B];  // wgrad: k row of the chunk, for the ragged-end mask
     const bf16_t* Ab = p.A;
     const bf16_t* Bb = p.B;
+    // Gated epilogue: the tile's row scales wait in LDS.  Loading them in the epilogue would put
+    // a vector load between the stores, and a load result can only be awaited together with
+    // every store issued before it.
+    __shared__ float s_rs[EPI == EPI_GATED ? BM : 1];
+    float rs_in = 1.0f;
+    if (EPI == EPI_GATED && tid < BM && p.row_scale) rs_in = p.row_scale[min(m0 + tid, mend - 1)];
 #pragma unroll
     for (int i = 0; i < PER_A; ++i) {
         const int c = tid + NT * i;
@@ -208,7 +236,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             a_kr[i] = 0;
         } else {
             constexpr int CPR = BM / 8;
-            const int krow = c / CPR, mc = (c % CPR) ^ (((krow >> 3) & 1) << 3);
+            const int krow = c / CPR, mc = (c % CPR) ^ ((krow & 3) << 2);
             const int col = min(m0 + mc * 8, p.M - 8);
             aoff[i] = A_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.lda + col;
             a_kr[i] = krow;
@@ -218,21 +246,19 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     for (int i = 0; i < PER_B; ++i) {
         const int c = tid + NT * i;
         if (B_KC) {
-            // LDS row slot s of a 64-row block holds column 2*(s%32) + s/32 of that block, so the
-            // even columns (one MFMA tile) and the odd columns (its partner) are each 32
-            // consecutive LDS rows
             const int row = c >> 2, kc = (c & 3) ^ ((row >> 2) & 3);
-            const int gn = min(n0 + (row & ~63) + 2 * (row & 31) + ((row >> 5) & 1), p.N - 1);
+            const int gn = min(n0 + row, p.N - 1);
             boff[i] = (uint32_t)gn * (uint32_t)p.ldb + kc * 8;
             b_kr[i] = 0;
         } else {
             constexpr int CPR = BN / 8;
-            const int krow = c / CPR, nc = (c % CPR) ^ (((krow >> 3) & 1) << 3);
+            const int krow = c / CPR, nc = (c % CPR) ^ ((krow & 3) << 2);
             const int col = min(n0 + nc * 8, p.N - 8);
             boff[i] = B_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.ldb + col;
             b_kr[i] = krow;
         }
     }
+    if (EPI == EPI_GATED && tid < BM) s_rs[tid] = rs_in;
     if (!WGRAD) {
         Bb += (long long)e * p.strideB;
     } else {
@@ -242,18 +268,50 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     const int k_rows = r1 - r0;  // wgrad: rows of this expert
 
     // Gathered operands of the weight gradient: the source row of a chunk changes with every K
-    // tile, so it is looked up one tile ahead (a_nxt / b_nxt, fetched right before the loads of
-    // the previous tile are issued) and moved to a_use / b_use when its own loads go out.
-    int a_use[PER_A], a_nxt[PER_A], b_use[PER_B], b_nxt[PER_B];
-    auto fetch_a_idx = [&](int kt, int (&dst)[PER_A]) {
+    // tile.  One wave-wide load covers RPW consecutive k rows starting at a wave-uniform row, so
+    // the row indices are fetched with SCALAR loads (their own counter: a vector load here would
+    // have to be awaited together with every direct-to-LDS load issued before it; the maps are
+    // only ever read by this kernel, which is what a scalar load requires) into a_snx /
+    // b_snx one tile ahead, and spread to the lanes (a_use / b_use) right after the fragment
+    // wait at the start of the step whose loads use them.
+    constexpr int RPW_A = 64 / (BM / 8), RPW_B = 64 / (BN / 8);
+    int a_use[PER_A], b_use[PER_B];
+    int a_snx[PER_A][RPW_A], b_snx[PER_B][RPW_B];
+    auto sfetch_a = [&](int kt, int (&dst)[PER_A][RPW_A]) {
 #pragma unroll
-        for (int i = 0; i < PER_A; ++i) dst[i] = p.a_row_map[min(r0 + kt * BK + a_kr[i], p.rows_total - 1)];
+        for (int i = 0; i < PER_A; ++i)
+#pragma unroll
+            for (int q = 0; q < RPW_A; ++q)
+                dst[i][q] = scalar_load_i32(p.a_row_map + min(r0 + kt * BK + (wave * 64 + NT * i) / (BM / 8) + q, p.rows_total - 1));
     };
-    auto fetch_b_idx = [&](int kt, int (&dst)[PER_B]) {
+    auto sfetch_b = [&](int kt, int (&dst)[PER_B][RPW_B]) {
 #pragma unroll
-        for (int i = 0; i < PER_B; ++i) dst[i] = p.b_row_map[min(r0 + kt * BK + b_kr[i], p.rows_total - 1)];
+        for (int i = 0; i < PER_B; ++i)
+#pragma unroll
+            for (int q = 0; q < RPW_B; ++q)
+                dst[i][q] = scalar_load_i32(p.b_row_map + min(r0 + kt * BK + (wave * 64 + NT * i) / (BN / 8) + q, p.rows_total - 1));
+    };
+    auto spread_a = [&](const int (&src)[PER_A][RPW_A], int (&dst)[PER_A]) {
+#pragma unroll
+        for (int i = 0; i < PER_A; ++i) {
+            int v = src[i][0];
+#pragma unroll
+            for (int q = 1; q < RPW_A; ++q) v = (lane / (BM / 8) == q) ? src[i][q] : v;
+            dst[i] = v;
+        }
+    };
+    auto spread_b = [&](const int (&src)[PER_B][RPW_B], int (&dst)[PER_B]) {
+#pragma unroll
+        for (int i = 0; i < PER_B; ++i) {
+            int v = src[i][0];
+#pragma unroll
+            for (int q = 1; q < RPW_B; ++q) v = (lane / (BN / 8) == q) ? src[i][q] : v;
+            dst[i] = v;
+        }
     };
 
+    const bf16_t* zero_src = reinterpret_cast<const bf16_t*>(g_zero_chunk);
+    asm volatile("" : "+s"(zero_src));  // keep the address in registers (not re-derived per load)
     // wgrad: rows past the end of the expert read a block of zeros instead (only the last K
     // tile of an expert can be ragged, the select costs two VALU ops per load)
     auto dma_a = [&](int kt, auto LO, auto HI, const int (&idx)[PER_A]) {
@@ -265,7 +323,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         for (int i = lo; i < hi; ++i) {
             const bf16_t* src = a_base + aoff[i];
             if (A_MAP) src += (long long)idx[i] * p.lda;
-            if (WGRAD) src = (k0 + a_kr[i] < k_rows) ? src : reinterpret_cast<const bf16_t*>(g_zero_chunk);
+            if (WGRAD) src = (k0 + a_kr[i] < k_rows) ? src : zero_src;
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sa + NT * i), 16, 0, 0);
         }
     };
@@ -278,27 +336,12 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         for (int i = lo; i < hi; ++i) {
             const bf16_t* src = b_base + boff[i];
             if (B_MAP) src += (long long)idx[i] * p.ldb;
-            if (WGRAD) src = (k0 + b_kr[i] < k_rows) ? src : reinterpret_cast<const bf16_t*>(g_zero_chunk);
+            if (WGRAD) src = (k0 + b_kr[i] < k_rows) ? src : zero_src;
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sb + NT * i), 16, 0, 0);
         }
     };
-    // steady-state issue: rotate the looked-up rows when the first half of a tile goes out
-    auto issue_a = [&](int kt, auto LO, auto HI) {
-        if (A_MAP && decltype(LO)::value == 0) {
-#pragma unroll
-            for (int i = 0; i < PER_A; ++i) a_use[i] = a_nxt[i];
-            fetch_a_idx(kt + 1, a_nxt);
-        }
-        dma_a(kt, LO, HI, a_use);
-    };
-    auto issue_b = [&](int kt, auto LO, auto HI) {
-        if (B_MAP && decltype(LO)::value == 0) {
-#pragma unroll
-            for (int i = 0; i < PER_B; ++i) b_use[i] = b_nxt[i];
-            fetch_b_idx(kt + 1, b_nxt);
-        }
-        dma_b(kt, LO, HI, b_use);
-    };
+    auto issue_a = [&](int kt, auto LO, auto HI) { dma_a(kt, LO, HI, a_use); };
+    auto issue_b = [&](int kt, auto LO, auto HI) { dma_b(kt, LO, HI, b_use); };
 
     mfma_f32x16 acc[TM][TN];
 #pragma unroll
@@ -309,79 +352,69 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     // ------------------------------------------------------------ fragment readers
-    // "raw" fragments are what comes out of LDS: for a K-contiguous operand the MFMA operand
-    // itself, for a K-strided operand eight dwords per tile pair still to be split by v_perm.
-    constexpr int RAW_A = A_KC ? TM : TM * 2;   // u32x4 registers
-    constexpr int RAW_B = B_KC ? TN : TN * 2;
-    auto read_a = [&](const u32x4_t* sa, int ks, u32x4_t (&ra)[RAW_A]) {
-        if (A_KC) {
+    // One 16-byte register quad per 32-wide tile and 16-deep K step, whatever the layout.
+    // K-strided operands: lane -> (k row, 4 columns) inside the 4x16 block its 16-lane group
+    // transposes; groups 0/1 take columns 0-15 / 16-31 of the tile, groups 2/3 the k rows 8-15.
+    // The transposing read is issued as inline assembly: through the builtin the compiler treats
+    // it as possibly aliasing the direct-to-LDS loads in flight and drains them all (vmcnt(0))
+    // before every read.  The compiler therefore does not track these reads; settle() below
+    // waits for them and ties the fragments to the wait.
+    const int tr_j = lane & 15, tr_blk = lane >> 4;
+    const int tr_col = 16 * (tr_blk & 1) + 4 * (tr_j & 3);   // first of this lane's 4 columns in the tile
+    const int tr_k = 8 * (tr_blk >> 1) + (tr_j >> 2);        // its k row inside the K step (+4 for the second read)
+    auto read_tr = [&](const u32x4_t* st, auto CPR_, int col0, auto KS) -> u32x4_t {
+        constexpr int cpr = decltype(CPR_)::value, ks = decltype(KS)::value;
+        const int col = col0 + tr_col;
+        const int chunk = (col >> 3) ^ ((tr_j >> 2) << 2);
+        const uint32_t addr = (uint32_t)(uintptr_t)(lptr_t)st + (uint32_t)((tr_k * cpr + chunk) * 16 + (col & 7) * 2);
+        u32x2_t lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(addr), "i"(ks * 16 * cpr * 16));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "i"((ks * 16 + 4) * cpr * 16));
+        return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+    };
+    auto read_a = [&](const u32x4_t* sa, auto KS, mfma_bf16x8 (&fa)[TM]) {
+        constexpr int ks = decltype(KS)::value;
 #pragma unroll
-            for (int t = 0; t < TM; ++t) {
+        for (int t = 0; t < TM; ++t) {
+            u32x4_t r;
+            if (A_KC) {
                 const int row = wm * WTM + t * 32 + lj;
                 const int kc = ks * 2 + lg;
-                ra[t] = sa[row * 4 + (kc ^ ((row >> 2) & 3))];
+                r = sa[row * 4 + (kc ^ ((row >> 2) & 3))];
+            } else {
+                r = read_tr(sa, std::integral_constant<int, BM / 8>{}, wm * WTM + t * 32, KS);
             }
-        } else {
-            constexpr int CPR = BM / 8;
-            const uint32_t* sw = reinterpret_cast<const uint32_t*>(sa);
-#pragma unroll
-            for (int pr = 0; pr < TM / 2; ++pr) {
-                const int word = (wm * WTM + pr * 64) / 2 + lj;
-                const int chunk = (word >> 2) ^ (lg << 3);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int krow = ks * 16 + lg * 8 + i;
-                    ra[pr * 2 + (i >> 2)][i & 3] = sw[(krow * CPR + chunk) * 4 + (word & 3)];
-                }
-            }
+            fa[t] = __builtin_bit_cast(mfma_bf16x8, r);
         }
     };
-    auto read_b = [&](const u32x4_t* sb, int ks, u32x4_t (&rb)[RAW_B]) {
-        if (B_KC) {
+    auto read_b = [&](const u32x4_t* sb, auto KS, mfma_bf16x8 (&fb)[TN]) {
+        constexpr int ks = decltype(KS)::value;
 #pragma unroll
-            for (int t = 0; t < TN; ++t) {
+        for (int t = 0; t < TN; ++t) {
+            u32x4_t r;
+            if (B_KC) {
                 const int row = wn * WTN + t * 32 + lj;
                 const int kc = ks * 2 + lg;
-                rb[t] = sb[row * 4 + (kc ^ ((row >> 2) & 3))];
+                r = sb[row * 4 + (kc ^ ((row >> 2) & 3))];
+            } else {
+                r = read_tr(sb, std::integral_constant<int, BN / 8>{}, wn * WTN + t * 32, KS);
             }
-        } else {
-            constexpr int CPR = BN / 8;
-            const uint32_t* sw = reinterpret_cast<const uint32_t*>(sb);
-#pragma unroll
-            for (int pr = 0; pr < TN / 2; ++pr) {
-                const int word = (wn * WTN + pr * 64) / 2 + lj;
-                const int chunk = (word >> 2) ^ (lg << 3);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int krow = ks * 16 + lg * 8 + i;
-                    rb[pr * 2 + (i >> 2)][i & 3] = sw[(krow * CPR + chunk) * 4 + (word & 3)];
-                }
-            }
+            fb[t] = __builtin_bit_cast(mfma_bf16x8, r);
         }
     };
-    // raw -> MFMA operands (identity for K-contiguous operands)
-    auto to_frag_pair = [&](const u32x4_t& w03, const u32x4_t& w47, mfma_bf16x8& even, mfma_bf16x8& odd) {
-        u32x4_t lo = {perm_lo(w03[1], w03[0]), perm_lo(w03[3], w03[2]), perm_lo(w47[1], w47[0]), perm_lo(w47[3], w47[2])};
-        u32x4_t hi = {perm_hi(w03[1], w03[0]), perm_hi(w03[3], w03[2]), perm_hi(w47[1], w47[0]), perm_hi(w47[3], w47[2])};
-        even = __builtin_bit_cast(mfma_bf16x8, lo);
-        odd = __builtin_bit_cast(mfma_bf16x8, hi);
-    };
-    auto make_fa = [&](const u32x4_t (&ra)[RAW_A], mfma_bf16x8 (&fa)[TM]) {
-        if (A_KC) {
+    // Called before the first MFMA that consumes fragments fetched by read_tr: waits for this
+    // wave's LDS reads and makes the fragments depend on the wait (an MFMA is otherwise free to
+    // be scheduled ahead of it).
+    auto settle = [&](mfma_bf16x8 (&fa)[TM], mfma_bf16x8 (&fb)[TN]) {
+        if (A_KC && B_KC) return;
+        asm volatile("s_waitcnt lgkmcnt(0)");
+        if (!A_KC) {
 #pragma unroll
-            for (int t = 0; t < TM; ++t) fa[t] = __builtin_bit_cast(mfma_bf16x8, ra[t]);
-        } else {
-#pragma unroll
-            for (int pr = 0; pr < TM / 2; ++pr) to_frag_pair(ra[2 * pr], ra[2 * pr + 1], fa[2 * pr], fa[2 * pr + 1]);
+            for (int t = 0; t < TM; ++t) asm volatile("" : "+v"(fa[t]));
         }
-    };
-    auto make_fb = [&](const u32x4_t (&rb)[RAW_B], mfma_bf16x8 (&fb)[TN]) {
-        if (B_KC) {
+        if (!B_KC) {
 #pragma unroll
-            for (int t = 0; t < TN; ++t) fb[t] = __builtin_bit_cast(mfma_bf16x8, rb[t]);
-        } else {
-#pragma unroll
-            for (int pr = 0; pr < TN / 2; ++pr) to_frag_pair(rb[2 * pr], rb[2 * pr + 1], fb[2 * pr], fb[2 * pr + 1]);
+            for (int t = 0; t < TN; ++t) asm volatile("" : "+v"(fb[t]));
         }
     };
     // quarter Q of a K step's MFMAs (A tile outer, B tile inner)
@@ -408,8 +441,8 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     // so the direct-to-LDS loads trickle out evenly (the L1 path moves 64 bytes a clock, half of
     // what the MFMAs consume at full rate) and each has about two iterations to land.
     // A step is written as four chunks fenced by scheduling barriers, each pairing a quarter of
-    // the MFMAs with one kind of side work: A-fragment reads, B-fragment reads, loads, loads +
-    // the v_perm splitting of K-strided fragments for the next step.
+    // the MFMAs with one kind of side work: A-fragment reads, B-fragment reads, loads, loads.
+    // Fragments are double-buffered: a step's reads fill the set the other step consumes.
     constexpr int PER = PER_A + PER_B;
     static_assert(2 * PER + PER_A <= 63, "vmcnt is a 6-bit counter");
     using IC0 = std::integral_constant<int, 0>;
@@ -420,30 +453,31 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     using A_ALL = std::integral_constant<int, PER_A>;
     using B_HALF = std::integral_constant<int, (PER_B + 1) / 2>;
     using B_ALL = std::integral_constant<int, PER_B>;
-    u32x4_t ra[RAW_A], rb[RAW_B];
     mfma_bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
 
     // prologue: tiles 0..2 and the A half of tile 3 go out, tile 0 is awaited
     {
         // row lookups of the first four tiles go out together, ahead of their loads
-        int ia[NSTAGE][PER_A], ib[NSTAGE][PER_B];
+        int sa4[NSTAGE][PER_A][RPW_A], sb4[NSTAGE][PER_B][RPW_B];
 #pragma unroll
         for (int t = 0; t < NSTAGE; ++t) {
-            if (A_MAP) fetch_a_idx(t, ia[t]);
-            if (B_MAP) fetch_b_idx(t, ib[t]);
+            if (A_MAP) sfetch_a(t, sa4[t]);
+            if (B_MAP && t < NSTAGE - 1) sfetch_b(t, sb4[t]);
         }
+        if (A_MAP) sfetch_a(NSTAGE, a_snx);      // next A tile to go out in the loop is tile 4
+        if (B_MAP) sfetch_b(NSTAGE - 1, b_snx);  // next B tile is tile 3
 #pragma unroll
         for (int t = 0; t < NSTAGE - 1; ++t) {
             if (t < kt_count) {
-                dma_a(t, IC0{}, A_ALL{}, ia[t]);
-                dma_b(t, IC0{}, B_ALL{}, ib[t]);
+                if (A_MAP) spread_a(sa4[t], a_use);
+                if (B_MAP) spread_b(sb4[t], b_use);
+                dma_a(t, IC0{}, A_ALL{}, a_use);
+                dma_b(t, IC0{}, B_ALL{}, b_use);
             }
         }
-        if (kt_count > NSTAGE - 1) dma_a(NSTAGE - 1, IC0{}, A_ALL{}, ia[NSTAGE - 1]);
-        if (A_MAP) fetch_a_idx(NSTAGE, a_nxt);          // next A tile to go out is tile 4
-        if (B_MAP) {
-#pragma unroll
-            for (int i = 0; i < PER_B; ++i) b_nxt[i] = ib[NSTAGE - 1][i];  // next B tile is tile 3
+        if (kt_count > NSTAGE - 1) {
+            if (A_MAP) spread_a(sa4[NSTAGE - 1], a_use);
+            dma_a(NSTAGE - 1, IC0{}, A_ALL{}, a_use);
         }
     }
     if (kt_count > NSTAGE - 1) {
@@ -452,10 +486,8 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         lds_barrier<0>();
     }
     if (kt_count > 0) {
-        read_a(smem, 0, ra);
-        read_b(smem + A_CH, 0, rb);
-        make_fa(ra, fa0);
-        make_fb(rb, fb0);
+        read_a(smem, IC0{}, fa0);
+        read_b(smem + A_CH, IC0{}, fb0);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -467,38 +499,42 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         const u32x4_t* sa = smem + (kt & (NSTAGE - 1)) * STAGE;
         const u32x4_t* sb = sa + A_CH;
         // ---- step A: MFMAs on (fa0, fb0)
-        read_a(sa, 1, ra);
+        settle(fa0, fb0);
+        if (B_MAP && load_b) {
+            spread_b(b_snx, b_use);     // rows of tile kt+3, whose loads go out in this step
+            sfetch_b(kt + 4, b_snx);
+        }
+        read_a(sa, IC1{}, fa1);
         mma_quarter(fa0, fb0, IC0{});
         __builtin_amdgcn_sched_barrier(0);
-        read_b(sb, 1, rb);
+        read_b(sb, IC1{}, fb1);
         mma_quarter(fa0, fb0, IC1{});
         __builtin_amdgcn_sched_barrier(0);
         if (load_b) issue_b(kt + 3, IC0{}, B_HALF{});
         mma_quarter(fa0, fb0, IC2{});
         __builtin_amdgcn_sched_barrier(0);
         if (load_b) issue_b(kt + 3, B_HALF{}, B_ALL{});
-        make_fa(ra, fa1);
-        make_fb(rb, fb1);
         mma_quarter(fa0, fb0, IC3{});
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier<waitn>();
         __builtin_amdgcn_sched_barrier(0);
         // ---- step B: MFMAs on (fa1, fb1)
         const u32x4_t* na = smem + ((kt + 1) & (NSTAGE - 1)) * STAGE;
-        if (next) read_a(na, 0, ra);
+        settle(fa1, fb1);
+        if (A_MAP && load_a) {
+            spread_a(a_snx, a_use);     // rows of tile kt+4
+            sfetch_a(kt + 5, a_snx);
+        }
+        if (next) read_a(na, IC0{}, fa0);
         mma_quarter(fa1, fb1, IC0{});
         __builtin_amdgcn_sched_barrier(0);
-        if (next) read_b(na + A_CH, 0, rb);
+        if (next) read_b(na + A_CH, IC0{}, fb0);
         mma_quarter(fa1, fb1, IC1{});
         __builtin_amdgcn_sched_barrier(0);
         if (load_a) issue_a(kt + 4, IC0{}, A_HALF{});
         mma_quarter(fa1, fb1, IC2{});
         __builtin_amdgcn_sched_barrier(0);
         if (load_a) issue_a(kt + 4, A_HALF{}, A_ALL{});
-        if (next) {
-            make_fa(ra, fa0);
-            make_fb(rb, fb0);
-        }
         mma_quarter(fa1, fb1, IC3{});
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -515,44 +551,45 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     }
 
     // ------------------------------------------------------------ epilogue
-    if (!WGRAD) {
+    // Lane l of tile (i, j) holds column j*32 + l%32 for 16 rows; registers v, v+1 (v even) are
+    // rows r, r+1.  Lanes 2c and 2c+1 swap one value each, after which the even lane owns the
+    // packed columns (2c, 2c+1) of row r and the odd lane those of row r+1: 4-byte stores.
+    // Gated: that pair is (gate, up) of intermediate column c; a second swap between lanes l and
+    // l^2 over two row pairs packs two neighbouring intermediate columns of one row.
+    bf16_t* Cb = WGRAD ? p.C + (long long)e * p.strideC : p.C;
+    const int odd1 = lj & 1, odd2 = (lj >> 1) & 1;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = m0 + wm * WTM + i * 32 + 8 * (v >> 2) + 4 * lg + (v & 3);
-                if (row >= mend) continue;
-                float rs = 1.0f;
-                if (EPI == EPI_GATED && p.row_scale) rs = p.row_scale[row];
+        for (int j = 0; j < TN; ++j) {
+            const int pcol = n0 + wn * WTN + j * 32 + (lj & ~1);
+            const bool col_ok = pcol < p.N;
 #pragma unroll
-                for (int pr = 0; pr < TN / 2; ++pr) {
-                    const int col = n0 + wn * WTN + pr * 64 + 2 * lj;
-                    if (col >= p.N) continue;
-                    const uint32_t packed = pack_bf16x2(acc[i][2 * pr][v], acc[i][2 * pr + 1][v]);
+            for (int v = 0; v < 16; v += 4) {
+                const int rt = wm * WTM + i * 32 + 8 * (v >> 2) + 4 * lg;  // rows rt..rt+3 of the tile
+                uint32_t pk[2];
+                float h[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const float x0 = acc[i][j][v + 2 * u], x1 = acc[i][j][v + 2 * u + 1];
+                    const float got = lane_xor1(odd1 ? x0 : x1);
+                    pk[u] = odd1 ? pack_bf16x2(got, x1) : pack_bf16x2(x0, got);
+                    const int prow = m0 + rt + 2 * u + odd1;
                     if (EPI == EPI_GATED) {
-                        if (p.C) *reinterpret_cast<uint32_t*>(p.C + (size_t)row * p.ldc + col) = packed;
-                        const float gte = bf16_lo(packed), up = bf16_hi(packed);
-                        p.C2[(size_t)row * p.ldc2 + (col >> 1)] = (bf16_t)(rs * up * act_fwd<ACT>(gte));
+                        h[u] = s_rs[rt + 2 * u + odd1] * bf16_hi(pk[u]) * act_fwd<ACT>(bf16_lo(pk[u]));
+                        if (p.C && col_ok && prow < mend)
+                            *reinterpret_cast<uint32_t*>(p.C + (size_t)prow * p.ldc + pcol) = pk[u];
                     } else {
-                        *reinterpret_cast<uint32_t*>(p.C + (size_t)row * p.ldc + col) = packed;
+                        if (col_ok && prow < mend) *reinterpret_cast<uint32_t*>(Cb + (size_t)prow * p.ldc + pcol) = pk[u];
                     }
                 }
-            }
-        }
-    } else {
-        bf16_t* Ce = p.C + (long long)e * p.strideC;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = m0 + wm * WTM + (i >> 1) * 64 + 2 * (8 * (v >> 2) + 4 * lg + (v & 3)) + (i & 1);
-                if (row >= p.M) continue;
-#pragma unroll
-                for (int pr = 0; pr < TN / 2; ++pr) {
-                    const int col = n0 + wn * WTN + pr * 64 + 2 * lj;
-                    if (col >= p.N) continue;
-                    *reinterpret_cast<uint32_t*>(Ce + (size_t)row * p.ldc + col) =
-                        pack_bf16x2(acc[i][2 * pr][v], acc[i][2 * pr + 1][v]);
+                if (EPI == EPI_GATED) {
+                    // lanes with bit 1 clear keep the first row pair, the others the second
+                    const float got = lane_xor2(odd2 ? h[0] : h[1]);
+                    const uint32_t hp = odd2 ? pack_bf16x2(got, h[1]) : pack_bf16x2(h[0], got);
+                    const int hrow = m0 + rt + 2 * odd2 + odd1;
+                    const int hcol = (pcol >> 1) & ~1;
+                    if (col_ok && hrow < mend) *reinterpret_cast<uint32_t*>(p.C2 + (size_t)hrow * p.ldc2 + hcol) = hp;
                 }
             }
         }
