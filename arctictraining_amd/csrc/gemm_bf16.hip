@@ -39,7 +39,8 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float mfma_f32x16;
 namespace {
 
 constexpr int BK = 32;      // K extent of one LDS stage
-constexpr int NSTAGE = 4;   // LDS stages in flight
+constexpr int NSTAGE = 4;   // LDS stages: one being consumed, the others landed or in flight.  (5 stages fit
+                            // the 160 KB of LDS and were measured: no faster.)
 
 struct GemmArgs {
     const bf16_t* A;
@@ -219,10 +220,10 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     int a_kr[PER_A], b_kr[PER_B];  // wgrad: k row of the chunk, for the ragged-end mask
     const bf16_t* Ab = p.A;
     const bf16_t* Bb = p.B;
-    // Gated epilogue: the tile's row scales wait in LDS.  Loading them in the epilogue would put
-    // a vector load between the stores, and a load result can only be awaited together with
-    // every store issued before it.
-    __shared__ float s_rs[EPI == EPI_GATED ? BM : 1];
+    // Gated epilogue: thread r < BM fetches the scale of tile row r now and parks it in LDS once
+    // the main loop has released the stages.  Loading the scales in the epilogue would put
+    // vector loads between the stores, and a load result can only be awaited together with every
+    // store issued before it.
     float rs_in = 1.0f;
     if (EPI == EPI_GATED && tid < BM && p.row_scale) rs_in = p.row_scale[min(m0 + tid, mend - 1)];
 #pragma unroll
@@ -258,7 +259,6 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             b_kr[i] = krow;
         }
     }
-    if (EPI == EPI_GATED && tid < BM) s_rs[tid] = rs_in;
     if (!WGRAD) {
         Bb += (long long)e * p.strideB;
     } else {
@@ -317,7 +317,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     auto dma_a = [&](int kt, auto LO, auto HI, const int (&idx)[PER_A]) {
         constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
         const int k0 = kt * BK;
-        u32x4_t* sa = smem + (kt & (NSTAGE - 1)) * STAGE + wave * 64;
+        u32x4_t* sa = smem + (kt % NSTAGE) * STAGE + wave * 64;
         const bf16_t* a_base = A_KC ? Ab + k0 : (A_MAP ? Ab : Ab + (long long)k0 * p.lda);
 #pragma unroll
         for (int i = lo; i < hi; ++i) {
@@ -330,7 +330,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     auto dma_b = [&](int kt, auto LO, auto HI, const int (&idx)[PER_B]) {
         constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
         const int k0 = kt * BK;
-        u32x4_t* sb = smem + (kt & (NSTAGE - 1)) * STAGE + A_CH + wave * 64;
+        u32x4_t* sb = smem + (kt % NSTAGE) * STAGE + A_CH + wave * 64;
         const bf16_t* b_base = B_KC ? Bb + k0 : (B_MAP ? Bb : Bb + (long long)k0 * p.ldb);
 #pragma unroll
         for (int i = lo; i < hi; ++i) {
@@ -430,8 +430,8 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     };
 
     // ------------------------------------------------------------ main loop
-    // NSTAGE = 4 LDS stages of one 32-wide K tile each (two MFMA K steps).  Iteration j works
-    // on tile j (stage j % 4):
+    // NSTAGE LDS stages of one 32-wide K tile each (two MFMA K steps); the offsets below are
+    // those of NSTAGE = 4.  Iteration j works on tile j (stage j % 4):
     //   step A: MFMAs on the ks=0 fragments | fetch the ks=1 fragments of tile j
     //           | issue the B half of the loads of tile j+3
     //   wait until tile j+1 has landed (the loads of tiles j+2, j+3 may stay in flight), barrier:
@@ -444,7 +444,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     // the MFMAs with one kind of side work: A-fragment reads, B-fragment reads, loads, loads.
     // Fragments are double-buffered: a step's reads fill the set the other step consumes.
     constexpr int PER = PER_A + PER_B;
-    static_assert(2 * PER + PER_A <= 63, "vmcnt is a 6-bit counter");
+    static_assert((NSTAGE - 2) * PER + PER_A <= 63, "vmcnt is a 6-bit counter");
     using IC0 = std::integral_constant<int, 0>;
     using IC1 = std::integral_constant<int, 1>;
     using IC2 = std::integral_constant<int, 2>;
@@ -464,8 +464,8 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             if (A_MAP) sfetch_a(t, sa4[t]);
             if (B_MAP && t < NSTAGE - 1) sfetch_b(t, sb4[t]);
         }
-        if (A_MAP) sfetch_a(NSTAGE, a_snx);      // next A tile to go out in the loop is tile 4
-        if (B_MAP) sfetch_b(NSTAGE - 1, b_snx);  // next B tile is tile 3
+        if (A_MAP) sfetch_a(NSTAGE, a_snx);      // next A tile to go out in the loop
+        if (B_MAP) sfetch_b(NSTAGE - 1, b_snx);  // next B tile to go out in the loop
 #pragma unroll
         for (int t = 0; t < NSTAGE - 1; ++t) {
             if (t < kt_count) {
@@ -481,13 +481,9 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         }
     }
     if (kt_count > NSTAGE - 1) {
-        lds_barrier<2 * PER + PER_A>();
+        lds_barrier<(NSTAGE - 2) * PER + PER_A>();
     } else {
         lds_barrier<0>();
-    }
-    if (kt_count > 0) {
-        read_a(smem, IC0{}, fa0);
-        read_b(smem + A_CH, IC0{}, fb0);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -496,13 +492,13 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         constexpr bool load_b = decltype(LOAD_B)::value, load_a = decltype(LOAD_A)::value;
         constexpr bool next = decltype(NEXT)::value;
         constexpr int waitn = decltype(WAITN)::value;
-        const u32x4_t* sa = smem + (kt & (NSTAGE - 1)) * STAGE;
+        const u32x4_t* sa = smem + (kt % NSTAGE) * STAGE;
         const u32x4_t* sb = sa + A_CH;
         // ---- step A: MFMAs on (fa0, fb0)
         settle(fa0, fb0);
         if (B_MAP && load_b) {
-            spread_b(b_snx, b_use);     // rows of tile kt+3, whose loads go out in this step
-            sfetch_b(kt + 4, b_snx);
+            spread_b(b_snx, b_use);     // rows of the B tile whose loads go out in this step
+            sfetch_b(kt + NSTAGE, b_snx);
         }
         read_a(sa, IC1{}, fa1);
         mma_quarter(fa0, fb0, IC0{});
@@ -510,20 +506,20 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         read_b(sb, IC1{}, fb1);
         mma_quarter(fa0, fb0, IC1{});
         __builtin_amdgcn_sched_barrier(0);
-        if (load_b) issue_b(kt + 3, IC0{}, B_HALF{});
+        if (load_b) issue_b(kt + NSTAGE - 1, IC0{}, B_HALF{});
         mma_quarter(fa0, fb0, IC2{});
         __builtin_amdgcn_sched_barrier(0);
-        if (load_b) issue_b(kt + 3, B_HALF{}, B_ALL{});
+        if (load_b) issue_b(kt + NSTAGE - 1, B_HALF{}, B_ALL{});
         mma_quarter(fa0, fb0, IC3{});
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier<waitn>();
         __builtin_amdgcn_sched_barrier(0);
         // ---- step B: MFMAs on (fa1, fb1)
-        const u32x4_t* na = smem + ((kt + 1) & (NSTAGE - 1)) * STAGE;
+        const u32x4_t* na = smem + ((kt + 1) % NSTAGE) * STAGE;
         settle(fa1, fb1);
         if (A_MAP && load_a) {
-            spread_a(a_snx, a_use);     // rows of tile kt+4
-            sfetch_a(kt + 5, a_snx);
+            spread_a(a_snx, a_use);     // rows of the A tile whose loads go out in this step
+            sfetch_a(kt + NSTAGE + 1, a_snx);
         }
         if (next) read_a(na, IC0{}, fa0);
         mma_quarter(fa1, fb1, IC0{});
@@ -531,23 +527,34 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         if (next) read_b(na + A_CH, IC0{}, fb0);
         mma_quarter(fa1, fb1, IC1{});
         __builtin_amdgcn_sched_barrier(0);
-        if (load_a) issue_a(kt + 4, IC0{}, A_HALF{});
+        if (load_a) issue_a(kt + NSTAGE, IC0{}, A_HALF{});
         mma_quarter(fa1, fb1, IC2{});
         __builtin_amdgcn_sched_barrier(0);
-        if (load_a) issue_a(kt + 4, A_HALF{}, A_ALL{});
+        if (load_a) issue_a(kt + NSTAGE, A_HALF{}, A_ALL{});
         mma_quarter(fa1, fb1, IC3{});
         __builtin_amdgcn_sched_barrier(0);
     };
-    {
+    // Every path through this block ends in the final k_tile, whose first action waits for the
+    // fragment reads still outstanding: none is in flight when the epilogue reuses the registers.
+    if (kt_count > 0) {
+        // W<r>: loads younger than tile kt+1 when r tiles (kt included) remain and none is left to issue
         using W0 = std::integral_constant<int, 0>;
         using W1 = std::integral_constant<int, PER>;
         using W2 = std::integral_constant<int, 2 * PER>;
+        using WFULL = std::integral_constant<int, (NSTAGE - 2) * PER>;
+        static_assert(NSTAGE == 4 || NSTAGE == 5, "the drain below is written out for 4 or 5 stages");
+        read_a(smem, IC0{}, fa0);
+        read_b(smem + A_CH, IC0{}, fb0);
+        __builtin_amdgcn_sched_barrier(0);
         int kt = 0;
-        for (; kt + 4 < kt_count; ++kt) k_tile(T_{}, T_{}, W2{}, T_{}, kt);
-        if (kt + 4 == kt_count) { k_tile(T_{}, F_{}, W2{}, T_{}, kt); ++kt; }
+        for (; kt + NSTAGE < kt_count; ++kt) k_tile(T_{}, T_{}, WFULL{}, T_{}, kt);
+        if (kt + NSTAGE == kt_count) { k_tile(T_{}, F_{}, WFULL{}, T_{}, kt); ++kt; }
+        if (NSTAGE == 5) {
+            if (kt + 4 == kt_count) { k_tile(F_{}, F_{}, W2{}, T_{}, kt); ++kt; }
+        }
         if (kt + 3 == kt_count) { k_tile(F_{}, F_{}, W1{}, T_{}, kt); ++kt; }
         if (kt + 2 == kt_count) { k_tile(F_{}, F_{}, W0{}, T_{}, kt); ++kt; }
-        if (kt + 1 == kt_count) k_tile(F_{}, F_{}, W0{}, F_{}, kt);
+        k_tile(F_{}, F_{}, W0{}, F_{}, kt);  // kt + 1 == kt_count here, whichever way it was reached
     }
 
     // ------------------------------------------------------------ epilogue
@@ -558,6 +565,12 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     // l^2 over two row pairs packs two neighbouring intermediate columns of one row.
     bf16_t* Cb = WGRAD ? p.C + (long long)e * p.strideC : p.C;
     const int odd1 = lj & 1, odd2 = (lj >> 1) & 1;
+    float* s_rs = reinterpret_cast<float*>(smem);   // the stages are free once every wave is past the loop
+    if (EPI == EPI_GATED) {
+        __syncthreads();
+        if (tid < BM) s_rs[tid] = rs_in;
+        __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -650,6 +663,12 @@ static int set_supertiles(GemmArgs& a, long long m_tiles, long long* grid)
 {
     a.gn = a.n_ntiles < 8 ? a.n_ntiles : 8;
     a.gm = 32 / a.gn;
+    // weight gradient: when all tiles of one expert fit in two rounds of an XCD's 32 CUs, the
+    // expert is the super-tile, so its rows are fetched into one L2 only
+    if (a.n_mt > 0 && (long long)a.n_mt * a.n_ntiles <= 64) {
+        a.gm = a.n_mt;
+        a.gn = a.n_ntiles;
+    }
     a.sn = (a.n_ntiles + a.gn - 1) / a.gn;
     const long long sm = (m_tiles + a.gm - 1) / a.gm;
     const long long supers = sm * a.sn;

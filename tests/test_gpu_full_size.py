@@ -1,0 +1,202 @@
+"""The BASELINE configurations at their FULL sizes.
+
+The float64 oracle cannot evaluate 3.7-17 TFLOP layers in seconds, so at full size the layer is
+checked through what does not grow with the size:
+  * routing -- top-k indices, counts, permutation maps -- bit-exact against the oracle on ALL
+    tokens (integer work, cheap on the CPU);
+  * y and dx of a handful of sampled tokens against the oracle run on just those tokens (with
+    loss_coeff = 0 a token's output and input gradient depend on no other token);
+  * sampled rows / columns of the expert weight gradients against their definition (the stage
+    formulas of the backward: dW_down[e][i,:] = sum_r inter_s[r,i] dy[tok_r,:], dW_gate_up[e][:,c]
+    = sum_r x[tok_r,:] d_gate_up[r,c]) evaluated in float64 over exactly the rows of that expert.
+C4 has no router: its grouped GEMMs are checked on sampled rows and elements the same way.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import moe_oracle as O
+from test_gpu_layer import build_layer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(gpu_device):
+    from arctictraining_amd import ops as _ops
+
+    return _ops
+
+
+TOL = 1e-2  # rel-L2, bf16
+
+# name: (T, H, E, K, I, bias_hot, n_hot, n_dead, oracle compute dtype)
+FULL = {
+    "c3_qwen3_30b": (16384, 2048, 128, 8, 768, None, 0, 0, torch.float64),
+    "c5_stress": (32768, 2048, 64, 4, 1408, 1.6, 4, 8, torch.float64),
+    "c2_mixtral": (8192, 4096, 8, 2, 14336, None, 0, 0, torch.float32),
+}
+
+
+def device_inputs(T, H, E, I, dev, seed, bias_hot=None, n_hot=0, n_dead=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    bf = torch.bfloat16
+    x = torch.randn(T, H, device=dev, generator=g)
+    wr = torch.randn(E, H, device=dev, generator=g) * 0.02
+    if n_hot or n_dead:
+        x[:, H - 1] = 1.0
+        wr[:, H - 1] = 0.0
+        wr[:n_hot, H - 1] = float(bias_hot)
+        wr[E - n_dead:, H - 1] = -1.0e4
+    x, wr = x.to(bf), wr.to(bf)
+    wgu = torch.empty(E, H, 2 * I, device=dev, dtype=bf)
+    wd = torch.empty(E, I, H, device=dev, dtype=bf)
+    for e in range(E):  # expert by expert: no float32 copy of the whole weight
+        wgu[e] = (torch.randn(H, 2 * I, device=dev, generator=g) * 0.02).to(bf)
+        wd[e] = (torch.randn(I, H, device=dev, generator=g) * 0.02).to(bf)
+    dy = torch.randn(T, H, device=dev, generator=g).to(bf)
+    return x, wr, wgu, wd, dy
+
+
+def bf16_round(t):
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
+@pytest.mark.parametrize("name", list(FULL))
+def test_full_size_layer(gpu_device, name):
+    T, H, E, K, I, bias_hot, n_hot, n_dead, odt = FULL[name]
+    print("full-size layer", name, flush=True)
+    dev = gpu_device
+    x, wr, wgu, wd, dy = device_inputs(T, H, E, I, dev, 4242, bias_hot, n_hot, n_dead)
+    layer = build_layer(torch.bfloat16, H, E, K, I, dev, loss_coeff=0.0)
+    with torch.no_grad():
+        layer.router_gate.copy_(wr)
+        layer.expert_gate_up.copy_(wgu)
+        layer.expert_down.copy_(wd)
+    layer.capture = {}
+    xg = x.clone().requires_grad_(True)
+    y = layer(xg)
+    y.backward(dy)
+    torch.cuda.synchronize()
+    cap = layer.capture
+
+    # ---- routing, all tokens, bit-exact
+    logits = cap["logits"].float().cpu()
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.0)
+    g = O.gate(logits, ocfg, torch.bfloat16, select_values=logits)
+    assert torch.equal(cap["topk_idx"].cpu().long(), g["topk_idx"]), "top-k indices"
+    assert torch.equal(cap["counts"].cpu().long(), g["counts"]), "counts"
+    assert torch.equal(cap["slot_of"].cpu().long(), g["perm"]), "permutation"
+    assert torch.equal(cap["token_of"].cpu().long(), g["token_ids"]), "token ids"
+    assert torch.equal(cap["row_of"].cpu().long(), O.inverse_row_map(g["perm"], T, K)), "inverse map"
+    # scores are floating point: equal up to one rounding step of the model dtype (2^-8 relative)
+    s_got, s_ref = cap["scores"].cpu().double(), g["scores_tk"].double()
+    assert float(((s_got - s_ref).abs() / s_ref).max()) <= 2.0 ** -7, "scores"
+    assert float((s_got != s_ref).double().mean()) < 0.01, "scores differ in more than 1% of the slots"
+    if n_dead:
+        assert int((g["counts"][-n_dead:] == 0).sum()) == n_dead
+        assert 0.35 < float(g["counts"][:n_hot].sum()) / float(g["counts"].sum()) < 0.65
+        assert bool((layer.expert_down.grad[-n_dead:] == 0).all()) and bool((layer.expert_gate_up.grad[-n_dead:] == 0).all())
+
+    # ---- sampled tokens against the oracle run on those tokens only
+    rng = np.random.default_rng(7)
+    S = torch.from_numpy(np.sort(rng.choice(T, size=16, replace=False)))
+    xs, dys = x[S.to(dev)].cpu(), dy[S.to(dev)].cpu()
+    ref = O.forward_backward(xs, wr.cpu(), wgu.cpu(), wd.cpu(), dys, ocfg, compute_dtype=odt,
+                             logits_for_selection=logits[S])
+    assert torch.equal(ref["topk_idx"], g["topk_idx"][S])
+    e_y = O.rel_l2(y.detach()[S.to(dev)].cpu(), ref["y"])
+    e_dx = O.rel_l2(xg.grad[S.to(dev)].cpu(), ref["dx"])
+    print(f"  sampled tokens: y {e_y:.2e} dx {e_dx:.2e}", flush=True)
+    assert e_y <= TOL and e_dx <= TOL
+    del ref
+
+    # ---- sampled rows / columns of the expert weight gradients against their definition
+    act, dact = O.activation("silu"), O.silu_grad
+    offsets = cap["offsets"].long()
+    token_of = cap["token_of"].long()
+    s_perm = cap["scores"].t().reshape(-1)[cap["slot_of"].long()].double()
+    counts = g["counts"]
+    live = [int(e) for e in torch.nonzero(counts > 0).flatten()]
+    experts = [live[0], live[len(live) // 2], live[-1]]
+    for e in experts:
+        r0, r1 = int(offsets[e]), int(offsets[e + 1])
+        tok = token_of[r0:r1]
+        Xe, DYe, se = x[tok].double(), dy[tok].double(), s_perm[r0:r1]
+        for i in (0, I // 2 + 1, I - 1):
+            gu = bf16_round(Xe @ wgu[e][:, 2 * i:2 * i + 2].double())           # stored in the model dtype
+            gate, up = gu[:, 0], gu[:, 1]
+            inter_s = bf16_round(se * up * act(gate))
+            ref_row = inter_s @ DYe                                            # dW_down[e][i, :]
+            err = O.rel_l2(layer.expert_down.grad[e, i].double(), ref_row)
+            assert err <= TOL, f"dW_down[{e}][{i}]: {err:.3e}"
+            d_inter = bf16_round(DYe @ wd[e][i].double())
+            d_gate = bf16_round(se * d_inter * up * dact(gate))
+            d_up = bf16_round(se * d_inter * act(gate))
+            for c, dcol in ((2 * i, d_gate), (2 * i + 1, d_up)):
+                ref_col = Xe.t() @ dcol                                        # dW_gate_up[e][:, c]
+                err = O.rel_l2(layer.expert_gate_up.grad[e, :, c].double(), ref_col)
+                assert err <= TOL, f"dW_gate_up[{e}][:, {c}]: {err:.3e}"
+
+
+def test_full_size_c4_grouped_gemms(ops, gpu_device):
+    """C4: one EP rank's share of a DeepSeek-V3-like layer -- 65536 pre-assigned rows,
+    32 local experts with Zipf(1.2) loads, H=7168, I=2048; forward and backward grouped GEMMs."""
+    R, E, H, I = 65536, 32, 7168, 2048
+    print("full-size c4", flush=True)
+    dev = gpu_device
+    rng = np.random.Generator(np.random.PCG64(44))
+    p = np.arange(1, E + 1, dtype=np.float64) ** -1.2
+    counts = rng.multinomial(R, p / p.sum())
+    offs_cpu = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    offs = torch.from_numpy(offs_cpu).to(dev)
+    g = torch.Generator(device=dev).manual_seed(44)
+    bf = torch.bfloat16
+    xp = torch.randn(R, H, device=dev, generator=g).to(bf)
+    dout = torch.randn(R, H, device=dev, generator=g).to(bf)
+    scores = torch.rand(R, device=dev, generator=g)
+    wgu = torch.empty(E, H, 2 * I, device=dev, dtype=bf)
+    wd = torch.empty(E, I, H, device=dev, dtype=bf)
+    for e in range(E):
+        wgu[e] = (torch.randn(H, 2 * I, device=dev, generator=g) * 0.02).to(bf)
+        wd[e] = (torch.randn(I, H, device=dev, generator=g) * 0.02).to(bf)
+    act, dact = O.activation("silu"), O.silu_grad
+
+    gate_up, inter_s = ops.grouped_gemm_gateup_act_fwd(xp, wgu, offs, row_scale=scores)
+    out = ops.grouped_gemm_nn(inter_s, wd, offs)
+    d_inter = ops.grouped_gemm_nt(dout, wd, offs)
+    d_wd = ops.grouped_gemm_wgrad(inter_s, dout, offs, E)
+    d_gu = ops.gated_act_bwd(gate_up, d_inter, row_scale=scores)
+    d_xp = ops.grouped_gemm_nt(d_gu, wgu, offs)
+    d_wgu = ops.grouped_gemm_wgrad(xp, d_gu, offs, E)
+    torch.cuda.synchronize()
+
+    expert_of = np.repeat(np.arange(E), counts)
+    rows = np.unique(np.concatenate([offs_cpu[:-1][counts > 0], offs_cpu[1:][counts > 0] - 1, rng.choice(R, 12)]))
+    for r in rows:
+        e = int(expert_of[r])
+        gu_ref = xp[r].double() @ wgu[e].double()
+        assert O.rel_l2(gate_up[r].double(), gu_ref) <= TOL, f"gate_up row {r}"
+        gu_b = gate_up[r].double()
+        inter_ref = scores[r].double() * gu_b[1::2] * act(gu_b[0::2])
+        assert O.rel_l2(inter_s[r].double(), inter_ref) <= TOL, f"inter row {r}"
+        assert O.rel_l2(out[r].double(), inter_s[r].double() @ wd[e].double()) <= TOL, f"down row {r}"
+        assert O.rel_l2(d_inter[r].double(), wd[e].double() @ dout[r].double()) <= TOL, f"d_inter row {r}"
+        dg_ref = torch.empty(2 * I, dtype=torch.float64, device=dev)
+        di = d_inter[r].double()
+        dg_ref[0::2] = scores[r].double() * di * gu_b[1::2] * dact(gu_b[0::2])
+        dg_ref[1::2] = scores[r].double() * di * act(gu_b[0::2])
+        assert O.rel_l2(d_gu[r].double(), dg_ref) <= TOL, f"d_gate_up row {r}"
+        assert O.rel_l2(d_xp[r].double(), wgu[e].double() @ d_gu[r].double()) <= TOL, f"d_xp row {r}"
+    for e in (0, E // 2, E - 1):
+        r0, r1 = int(offs_cpu[e]), int(offs_cpu[e + 1])
+        for i in (0, I - 1):
+            ref_row = inter_s[r0:r1, i].double() @ dout[r0:r1].double()
+            assert O.rel_l2(d_wd[e, i].double(), ref_row) <= TOL, f"dW_down[{e}][{i}]"
+        for c in (1, 2 * I - 2):
+            ref_col = xp[r0:r1].double().t() @ d_gu[r0:r1, c].double()
+            assert O.rel_l2(d_wgu[e, :, c].double(), ref_col) <= TOL, f"dW_gate_up[{e}][:, {c}]"
+    # rows are processed exactly once: every output row is written (no NaN / stale memory)
+    for t in (gate_up, inter_s, out, d_inter, d_xp, d_wd, d_wgu):
+        assert bool(torch.isfinite(t.float()).all())
