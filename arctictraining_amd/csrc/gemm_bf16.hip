@@ -559,10 +559,14 @@ grouped_gemm_bf16_kernel(GemmArgs p)
 
     // ------------------------------------------------------------ epilogue
     // Lane l of tile (i, j) holds column j*32 + l%32 for 16 rows; registers v, v+1 (v even) are
-    // rows r, r+1.  Lanes 2c and 2c+1 swap one value each, after which the even lane owns the
-    // packed columns (2c, 2c+1) of row r and the odd lane those of row r+1: 4-byte stores.
-    // Gated: that pair is (gate, up) of intermediate column c; a second swap between lanes l and
-    // l^2 over two row pairs packs two neighbouring intermediate columns of one row.
+    // rows r, r+1.  Each lane converts its two values to one packed bf16 pair, lanes 2c and 2c+1
+    // exchange the pairs (DPP) and a byte permute leaves the even lane with columns (2c, 2c+1) of
+    // row r and the odd lane with those of row r+1: three VALU operations per 4-byte store.
+    // Gated: that pair is (gate, up) of intermediate column c; a second exchange between lanes l
+    // and l^2 over two row pairs packs two neighbouring intermediate columns of one row.
+    // Addresses are a wave-uniform row base (scalar arithmetic) plus one per-lane 32-bit offset;
+    // tiles that lie entirely inside their expert's rows and the matrix take the FULL form
+    // without per-store bounds tests.
     bf16_t* Cb = WGRAD ? p.C + (long long)e * p.strideC : p.C;
     const int odd1 = lj & 1, odd2 = (lj >> 1) & 1;
     float* s_rs = reinterpret_cast<float*>(smem);   // the stages are free once every wave is past the loop
@@ -571,42 +575,55 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         if (tid < BM) s_rs[tid] = rs_in;
         __syncthreads();
     }
+    const uint32_t swap_sel = odd1 ? 0x03020706u : 0x05040100u;
+    // wave-uniform origin of this wave's part of the tile, and the lane's offset from it (bytes)
+    const long long worg = (long long)(m0 + wm * WTM) * p.ldc + n0 + wn * WTN;
+    const long long worg2 = (long long)(m0 + wm * WTM) * p.ldc2 + ((n0 + wn * WTN) >> 1);
+    char* cbase = reinterpret_cast<char*>((EPI == EPI_GATED ? p.C : Cb) + worg);
+    char* c2base = EPI == EPI_GATED ? reinterpret_cast<char*>(p.C2 + worg2) : nullptr;
+    const uint32_t loff = (uint32_t)((4 * lg + odd1) * p.ldc + (lj & ~1)) * 2u;
+    const uint32_t loff2 = EPI == EPI_GATED ? (uint32_t)((4 * lg + 2 * odd2 + odd1) * p.ldc2 + ((lj >> 1) & ~1)) * 2u : 0u;
+    const bool want_c = EPI != EPI_GATED || p.C != nullptr;
+    auto epilogue = [&](auto FULL) {
+        constexpr bool full = decltype(FULL)::value;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int pcol = n0 + wn * WTN + j * 32 + (lj & ~1);
-            const bool col_ok = pcol < p.N;
+            for (int j = 0; j < TN; ++j) {
+                const bool col_ok = full || (n0 + wn * WTN + j * 32 + (lj & ~1) < p.N);
 #pragma unroll
-            for (int v = 0; v < 16; v += 4) {
-                const int rt = wm * WTM + i * 32 + 8 * (v >> 2) + 4 * lg;  // rows rt..rt+3 of the tile
-                uint32_t pk[2];
-                float h[2];
+                for (int v = 0; v < 16; v += 4) {
+                    const int rq = i * 32 + 8 * (v >> 2);           // first of 8 rows, relative to the wave's origin
+                    const int rt = wm * WTM + rq + 4 * lg;          // rows rt..rt+3 of the tile
+                    float h[2];
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const float x0 = acc[i][j][v + 2 * u], x1 = acc[i][j][v + 2 * u + 1];
-                    const float got = lane_xor1(odd1 ? x0 : x1);
-                    pk[u] = odd1 ? pack_bf16x2(got, x1) : pack_bf16x2(x0, got);
-                    const int prow = m0 + rt + 2 * u + odd1;
-                    if (EPI == EPI_GATED) {
-                        h[u] = s_rs[rt + 2 * u + odd1] * bf16_hi(pk[u]) * act_fwd<ACT>(bf16_lo(pk[u]));
-                        if (p.C && col_ok && prow < mend)
-                            *reinterpret_cast<uint32_t*>(p.C + (size_t)prow * p.ldc + pcol) = pk[u];
-                    } else {
-                        if (col_ok && prow < mend) *reinterpret_cast<uint32_t*>(Cb + (size_t)prow * p.ldc + pcol) = pk[u];
+                    for (int u = 0; u < 2; ++u) {
+                        const uint32_t own = pack_bf16x2(acc[i][j][v + 2 * u], acc[i][j][v + 2 * u + 1]);
+                        const uint32_t got = __builtin_amdgcn_update_dpp(0, own, 0xB1, 0xF, 0xF, true);
+                        const uint32_t pk = __builtin_amdgcn_perm(got, own, swap_sel);
+                        const bool ok = full || (col_ok && m0 + rt + 2 * u + odd1 < mend);
+                        if (EPI == EPI_GATED)
+                            h[u] = s_rs[rt + 2 * u + odd1] * bf16_hi(pk) * act_fwd<ACT>(bf16_lo(pk));
+                        if (want_c && ok) {
+                            char* rowp = cbase + ((long long)(rq + 2 * u) * p.ldc + j * 32) * 2;
+                            *reinterpret_cast<uint32_t*>(rowp + loff) = pk;
+                        }
                     }
-                }
-                if (EPI == EPI_GATED) {
-                    // lanes with bit 1 clear keep the first row pair, the others the second
-                    const float got = lane_xor2(odd2 ? h[0] : h[1]);
-                    const uint32_t hp = odd2 ? pack_bf16x2(got, h[1]) : pack_bf16x2(h[0], got);
-                    const int hrow = m0 + rt + 2 * odd2 + odd1;
-                    const int hcol = (pcol >> 1) & ~1;
-                    if (col_ok && hrow < mend) *reinterpret_cast<uint32_t*>(p.C2 + (size_t)hrow * p.ldc2 + hcol) = hp;
+                    if (EPI == EPI_GATED) {
+                        // lanes with bit 1 clear keep the first row pair, the others the second
+                        const float got = lane_xor2(odd2 ? h[0] : h[1]);
+                        const uint32_t hp = odd2 ? pack_bf16x2(got, h[1]) : pack_bf16x2(h[0], got);
+                        const bool ok = full || (col_ok && m0 + rt + 2 * odd2 + odd1 < mend);
+                        if (ok) {
+                            char* rowp = c2base + ((long long)rq * p.ldc2 + j * 16) * 2;
+                            *reinterpret_cast<uint32_t*>(rowp + loff2) = hp;
+                        }
+                    }
                 }
             }
         }
-    }
+    };
+    if (m0 + BM <= mend && n0 + BN <= p.N) epilogue(T_{}); else epilogue(F_{});
 }
 
 // ------------------------------------------------------------------ host side
