@@ -91,6 +91,29 @@ class PhaseTimers:
         return self.times[name]
 
 
+_SPLIT_OFFSETS = {}
+
+
+def _router_weight_grad(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """dW_router [E,H] = d_logits^T [E,T] @ x [T,H] (autograd of moe.py:233).
+
+    The product is skinny (E rows) and deep (T): the library GEMM leaves most of the chip idle on
+    it.  For bf16 it is run as a split-K on the grouped weight-gradient kernel instead -- the
+    tokens are cut into chunks that play the role of experts, C[s] = d_logits[chunk s]^T @
+    x[chunk s] -- and the partial products are summed in float32."""
+    T, E = d_logits.shape
+    splits = 16
+    if x.dtype != torch.bfloat16 or E % 8 or T % (splits * 32):
+        return torch.matmul(d_logits.t(), x)
+    key = (T, splits, x.device)
+    offs = _SPLIT_OFFSETS.get(key)
+    if offs is None:
+        offs = torch.arange(0, T + 1, T // splits, dtype=torch.int32, device=x.device)
+        _SPLIT_OFFSETS[key] = offs
+    part = ops.grouped_gemm_wgrad(d_logits, x, offs, splits, tile_cfg=1)  # [splits, E, H], 128x128 tiles
+    return part.sum(dim=0, dtype=torch.float32).to(x.dtype)
+
+
 class _ExpertLayerFn(torch.autograd.Function):
     """router top-k -> permutation -> grouped gated FFN -> weighted combine, and the
     gradients of all of it (the autograd of moe.py:231-233, 340-411, 176-193, 450-461 plus
@@ -166,7 +189,7 @@ class _ExpertLayerFn(torch.autograd.Function):
         d_logits = ops.router_bwd(
             d_scores, probs, topk_idx, counts, x.dtype, opts["normalize"], opts["loss_coeff"] / T / opts["ep_size"]
         )
-        d_router_gate = torch.matmul(d_logits.t(), x) if ctx.needs_input_grad[1] else None
+        d_router_gate = _router_weight_grad(d_logits, x) if ctx.needs_input_grad[1] else None
         dx = None
         if ctx.needs_input_grad[0]:
             d_xp = ops.grouped_gemm_nt(d_gate_up, w_gate_up, offsets, tile_cfg=cfg)
