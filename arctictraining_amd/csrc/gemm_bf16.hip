@@ -678,11 +678,13 @@ int launch_any(const GemmArgs& a, int tile_cfg, int grid, hipStream_t s)
 // super-tile shape and grid size for `m_tiles` (upper bound) x `n_ntiles` tiles
 static int set_supertiles(GemmArgs& a, long long m_tiles, long long* grid)
 {
-    a.gn = a.n_ntiles < 8 ? a.n_ntiles : 8;
+    // at most 8 N tiles per super-tile, the N super-columns of equal width (11 -> 6 + 5, not 8 + 3)
+    const int n_super = (a.n_ntiles + 7) / 8;
+    a.gn = (a.n_ntiles + n_super - 1) / n_super;
     a.gm = 32 / a.gn;
-    // weight gradient: when all tiles of one expert fit in two rounds of an XCD's 32 CUs, the
+    // weight gradient: when all tiles of one expert fit in one round of an XCD's 32 CUs, the
     // expert is the super-tile, so its rows are fetched into one L2 only
-    if (a.n_mt > 0 && (long long)a.n_mt * a.n_ntiles <= 64) {
+    if (a.n_mt > 0 && (long long)a.n_mt * a.n_ntiles <= 32) {
         a.gm = a.n_mt;
         a.gn = a.n_ntiles;
     }
