@@ -58,6 +58,14 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
          _c_void_p],
     ),
+    "amoe_remap_pack": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, ctypes.c_longlong, _c_void_p],
+    ),
+    "amoe_remap_unpack": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, ctypes.c_longlong, _c_void_p],
+    ),
     "amoe_gated_act_bwd": (
         _c_int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,

@@ -18,7 +18,7 @@ OBJ_DIR = os.path.join(SRC_DIR, "build")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libarctic_moe_hip.so")
 
-SOURCES = ["api.hip", "router.hip", "permute.hip", "rows.hip", "gemm_bf16.hip", "gemm_f32.hip"]
+SOURCES = ["api.hip", "router.hip", "permute.hip", "rows.hip", "gemm_bf16.hip", "gemm_f32.hip", "remap.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

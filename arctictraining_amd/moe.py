@@ -50,7 +50,7 @@ def classify_activation(act_fn) -> int:
         return act_fn
     if isinstance(act_fn, str):
         return {"silu": ops.ACT_SILU, "gelu": ops.ACT_GELU, "relu": ops.ACT_RELU, "gpt_oss": ops.ACT_GPT_OSS}[act_fn]
-    probe = torch.tensor([-2.0, -0.5, 0.3, 1.7], dtype=torch.float32)
+    probe = torch.tensor([-2.0, -0.5, 0.3, 1.7], dtype=torch.float32, device="cpu")  # also under a meta-device context
     got = act_fn(probe)
     candidates = {
         ops.ACT_SILU: F.silu(probe),

@@ -290,3 +290,51 @@ def gated_act_bwd(
     )
     _lib.check(rc, "amoe_gated_act_bwd")
     return d_gu if slot_of is None else (d_gu, d_scale)
+
+
+def _expert_view(t: torch.Tensor, name: str):
+    """[E, I, H] tensor whose experts may be strided (a slice of a fused tensor) but whose
+    [I, H] matrices are dense; returns (E, I, H, expert stride in elements)."""
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (the HIP kernels have no CPU fallback)")
+    if t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != t.shape[2]:
+        raise RuntimeError(f"{name} must be [E, I, H] with dense [I, H] matrices, got strides {t.stride()}")
+    return t.shape[0], t.shape[1], t.shape[2], (t.stride(0) if t.shape[0] > 1 else t.shape[1] * t.shape[2])
+
+
+def remap_pack(in0: torch.Tensor, in1: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[e][h][G*i+g] = in_g[e][i][h]: gate/up nn.Linear weights [E,I,H] -> interleaved
+    expert_gate_up [E,H,2I] (in1 given), or a batched transpose [E,I,H] -> [E,H,I] (in1 None)."""
+    lib = _lib.load()
+    E, I, H, es = _expert_view(in0, "in0")
+    if in1 is not None:
+        if _expert_view(in1, "in1") != (E, I, H, es) or in1.dtype != in0.dtype:
+            raise RuntimeError("in1 must match in0 in shape, strides and dtype")
+    out = torch.empty((E, H, (2 if in1 is not None else 1) * I), dtype=in0.dtype, device=in0.device)
+    rc = lib.amoe_remap_pack(in0.data_ptr(), _ptr(in1), out.data_ptr(), _dtype_code(in0), E, I, H, es, _stream())
+    _lib.check(rc, "amoe_remap_pack")
+    return out
+
+
+def remap_unpack(joint: torch.Tensor, two: bool, out0: Optional[torch.Tensor] = None, out1: Optional[torch.Tensor] = None):
+    """The inverse of remap_pack: joint [E,H,G*I] -> out_g [E,I,H] (G = 2 if `two`).  out0 / out1
+    may be given (e.g. the halves of a fused [E,2I,H] tensor); returns out0 or (out0, out1)."""
+    lib = _lib.load()
+    _chk(joint, "joint")
+    E, H, GI = joint.shape
+    G = 2 if two else 1
+    if GI % G:
+        raise RuntimeError("the last dimension of an interleaved gate_up tensor must be even")
+    I = GI // G
+    if out0 is None:
+        out0 = torch.empty((E, I, H), dtype=joint.dtype, device=joint.device)
+        out1 = torch.empty((E, I, H), dtype=joint.dtype, device=joint.device) if two else None
+    shape = _expert_view(out0, "out0")
+    if shape[:3] != (E, I, H) or out0.dtype != joint.dtype:
+        raise RuntimeError("out0 must be [E, I, H] of the input's dtype")
+    if two and (out1 is None or _expert_view(out1, "out1") != shape or out1.dtype != joint.dtype):
+        raise RuntimeError("out1 must match out0")
+    rc = lib.amoe_remap_unpack(joint.data_ptr(), out0.data_ptr(), _ptr(out1) if two else None, _dtype_code(joint), E, I, H,
+                               shape[3], _stream())
+    _lib.check(rc, "amoe_remap_unpack")
+    return (out0, out1) if two else out0

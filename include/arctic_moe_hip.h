@@ -180,6 +180,28 @@ int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, const float* ro
                        void* d_gate_up, float* d_row_scale, int dtype, int R, int I, int T, int K, int act,
                        void* stream);
 
+/*
+ * Expert-weight re-layout, checkpoint format -> ArcticMoE parameters.  Replaces the torch
+ * stack / view / transpose sequence of remap_orig_moe_mlp_params_to_arctic_moe
+ * (arctic_training/model/moe/utils.py:232-266):
+ *   out[e][h][G*i + g] = in_g[e][i][h],   in_g [E, I, H] (nn.Linear weights, [out, in]),
+ * G = 2 when in1 is given (in0 = gate_proj, in1 = up_proj -> expert_gate_up [E, H, 2I] with
+ * gate in the even and up in the odd columns), G = 1 when in1 is null (down_proj [E, H', I']
+ * passed as I = H', H = I' -> expert_down: a batched transpose).  in_expert_stride is the
+ * distance in elements between experts of in0 / in1 (I*H when they are dense; 2*I*H when both
+ * are halves of one fused [E, 2I, H] tensor).  out is dense.  Bit-exact.
+ */
+int amoe_remap_pack(const void* in0, const void* in1, void* out, int dtype, int E, int I, int H,
+                    long long in_expert_stride, void* stream);
+
+/*
+ * The inverse, ArcticMoE parameters -> checkpoint format
+ * (remap_arctic_moe_to_orig_moe_mlp_params, utils.py:366-395):
+ *   out_g[e][i][h] = in[e][h][G*i + g],   G = 2 when out1 is given, else 1.
+ */
+int amoe_remap_unpack(const void* in, void* out0, void* out1, int dtype, int E, int I, int H,
+                      long long out_expert_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -103,6 +103,16 @@ def test_gemm_argument_errors(lib):
     assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, None, None, P, 0, 128, 4, 64, 64, 0, P, big, 0, None) == -2
 
 
+def test_remap_argument_errors(lib):
+    assert lib.amoe_remap_pack(None, P, P, 1, 2, 64, 64, 64 * 64, None) == -1
+    assert lib.amoe_remap_pack(P, P, P, 5, 2, 64, 64, 64 * 64, None) == -1  # dtype
+    assert lib.amoe_remap_pack(P, P, P, 1, 2, 60, 64, 60 * 64, None) == -2  # bf16 extents are multiples of 8
+    assert lib.amoe_remap_pack(P, P, P, 0, 2, 62, 64, 62 * 64, None) == -2  # float32: multiples of 4
+    assert lib.amoe_remap_pack(P, P, P, 1, 2, 64, 64, 100, None) == -1  # expert stride below I*H
+    assert lib.amoe_remap_unpack(P, None, P, 1, 2, 64, 64, 64 * 64, None) == -1
+    assert lib.amoe_remap_unpack(P, P, None, 1, 0, 64, 64, 64 * 64, None) == -1  # E
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libarctic_moe_hip.so")

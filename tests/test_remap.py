@@ -1,0 +1,206 @@
+"""Expert-weight re-layout (checkpoint format <-> ArcticMoE parameters).
+
+CPU part: the numpy oracle is pinned by element-by-element index loops, by the literal torch
+sequence the reference runs (utils.py:232-251 / 366-379), by round trips, and through the
+installed transformers Qwen3MoeSparseMoeBlock: its forward must equal the oracle's ArcticMoE
+forward on the weights the remap oracle packed.
+GPU part (marked gpu): the HIP kernels through the C ABI are bit-exact against the oracle,
+including ragged tile edges, fused [E,2I,H] inputs, float32, and the headline shape by round
+trip; the install / restore hooks reproduce the HF block's output and give its weights back
+bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from oracle import remap_oracle as RO
+
+
+def _rand(shape, seed):
+    return np.random.default_rng(seed).integers(0, 2**16, size=shape, dtype=np.uint16)
+
+
+def test_oracle_pack_matches_index_definition():
+    E, I, H = 2, 3, 5
+    gate, up, down = _rand((E, I, H), 1), _rand((E, I, H), 2), _rand((E, H, I), 3)
+    gu, dn = RO.pack_gate_up(gate, up), RO.pack_down(down)
+    assert gu.shape == (E, H, 2 * I) and dn.shape == (E, I, H)
+    for e in range(E):
+        for i in range(I):
+            for h in range(H):
+                assert gu[e, h, 2 * i] == gate[e, i, h]
+                assert gu[e, h, 2 * i + 1] == up[e, i, h]
+                assert dn[e, i, h] == down[e, h, i]
+
+
+def test_oracle_matches_reference_torch_sequence():
+    E, I, H = 3, 4, 6
+    g = torch.randn(E, I, H)
+    u = torch.randn(E, I, H)
+    # utils.py:232-247: per-expert `.weight.T` stacked, then stack(dim=-1).view
+    gate_stacked = torch.stack([g[i].T for i in range(E)])
+    up_stacked = torch.stack([u[i].T for i in range(E)])
+    ref = torch.stack((gate_stacked, up_stacked), dim=-1).view(*up_stacked.shape[:-1], -1).contiguous()
+    assert np.array_equal(RO.pack_gate_up(g.numpy(), u.numpy()), ref.numpy())
+    # utils.py:366-374: unbind of the (-1, 2) view
+    gate_un, up_un = torch.unbind(ref.view(-1, 2), dim=-1)
+    gate_un = gate_un.view(*ref.shape[:-1], -1)
+    g2, u2 = RO.unpack_gate_up(ref.numpy())
+    assert np.array_equal(g2, torch.stack([x.T for x in gate_un.unbind()]).numpy())
+    assert np.array_equal(g2, g.numpy()) and np.array_equal(u2, u.numpy())
+
+
+def test_oracle_round_trip():
+    E, I, H = 4, 24, 40
+    gate, up, down = _rand((E, I, H), 4), _rand((E, I, H), 5), _rand((E, H, I), 6)
+    g2, u2 = RO.unpack_gate_up(RO.pack_gate_up(gate, up))
+    assert np.array_equal(g2, gate) and np.array_equal(u2, up)
+    assert np.array_equal(RO.unpack_down(RO.pack_down(down)), down)
+
+
+def _tiny_hf_block(dtype=torch.float64, E=8, K=2, H=32, I=16, seed=0):
+    from transformers import Qwen3MoeConfig
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeSparseMoeBlock
+
+    c = Qwen3MoeConfig(
+        hidden_size=H, intermediate_size=4 * H, moe_intermediate_size=I, num_experts=E, num_experts_per_tok=K,
+        norm_topk_prob=True, num_hidden_layers=1, num_attention_heads=2, num_key_value_heads=2, vocab_size=64,
+        hidden_act="silu", router_aux_loss_coef=0.0,
+    )
+    torch.manual_seed(seed)
+    blk = Qwen3MoeSparseMoeBlock(c)
+    with torch.no_grad():
+        for p in blk.parameters():
+            p.copy_(torch.randn_like(p) * 0.2)
+    return c, blk.to(dtype)
+
+
+def test_packed_weights_reproduce_hf_block():
+    c, blk = _tiny_hf_block()
+    E, I, H = c.num_experts, c.moe_intermediate_size, c.hidden_size
+    fused = blk.experts.gate_up_proj.detach().numpy()
+    gu = torch.from_numpy(RO.pack_gate_up(fused[:, :I, :], fused[:, I:, :]))
+    dn = torch.from_numpy(RO.pack_down(blk.experts.down_proj.detach().numpy()))
+    x = torch.randn(2, 11, H, dtype=torch.float64)
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=c.num_experts_per_tok, loss_coeff=0.0)
+    ref = O.forward(x.view(-1, H), blk.gate.weight.detach(), gu, dn, ocfg, compute_dtype=torch.float64)
+    assert torch.allclose(ref["y"].view_as(x), blk(x), atol=5e-6)
+
+
+# ------------------------------------------------------------------ GPU: the HIP kernels
+@pytest.fixture(scope="module")
+def ops(gpu_device):
+    from arctictraining_amd import ops as _ops
+
+    return _ops
+
+
+def _as_np(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16) if t.dtype == torch.bfloat16 else t.cpu().numpy()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,E,I,H", [
+    (torch.bfloat16, 3, 64, 128), (torch.bfloat16, 2, 72, 200), (torch.bfloat16, 1, 8, 8),
+    (torch.bfloat16, 5, 192, 256), (torch.float32, 2, 36, 52), (torch.float32, 3, 128, 64),
+])
+def test_hip_remap_bit_exact(ops, gpu_device, dtype, E, I, H):
+    print("remap", dtype, E, I, H, flush=True)
+    g = torch.Generator().manual_seed(E * 1000 + I + H)
+    gate, up = torch.randn(E, I, H, generator=g).to(dtype), torch.randn(E, I, H, generator=g).to(dtype)
+    down = torch.randn(E, H, I, generator=g).to(dtype)
+    gu = ops.remap_pack(gate.to(gpu_device), up.to(gpu_device))
+    dn = ops.remap_pack(down.to(gpu_device))
+    assert np.array_equal(_as_np(gu), RO.pack_gate_up(_as_np(gate), _as_np(up)))
+    assert np.array_equal(_as_np(dn), RO.pack_down(_as_np(down)))
+    # fused [E, 2I, H] input: two strided halves of one tensor
+    fused = torch.cat((gate, up), dim=1).to(gpu_device)
+    assert torch.equal(ops.remap_pack(fused[:, :I, :], fused[:, I:, :]), gu)
+    # inverse
+    g2, u2 = ops.remap_unpack(gu, two=True)
+    assert torch.equal(g2.cpu(), gate) and torch.equal(u2.cpu(), up)
+    assert torch.equal(ops.remap_unpack(dn, two=False).cpu(), down)
+    out = torch.empty_like(fused)
+    ops.remap_unpack(gu, two=True, out0=out[:, :I, :], out1=out[:, I:, :])
+    assert torch.equal(out, fused)
+
+
+@pytest.mark.gpu
+def test_hip_remap_headline_shape_round_trip(ops, gpu_device):
+    E, I, H = 128, 768, 2048
+    g = torch.Generator(device=gpu_device).manual_seed(5)
+    fused = torch.randn(E, 2 * I, H, device=gpu_device, generator=g).to(torch.bfloat16)
+    gu = ops.remap_pack(fused[:, :I, :], fused[:, I:, :])
+    # sampled elements against the definition, then the whole tensor by round trip
+    rng = np.random.default_rng(3)
+    for e, i, h in zip(rng.integers(0, E, 64), rng.integers(0, I, 64), rng.integers(0, H, 64)):
+        assert gu[e, h, 2 * i] == fused[e, i, h] and gu[e, h, 2 * i + 1] == fused[e, I + i, h]
+    back = torch.empty_like(fused)
+    ops.remap_unpack(gu, two=True, out0=back[:, :I, :], out1=back[:, I:, :])
+    assert torch.equal(back, fused)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("as_list", [False, True])
+def test_install_and_restore_hooks(gpu_device, as_list):
+    """A one-layer stand-in for a HF MoE model: install ArcticMoE from its block, compare the
+    forward with the block's own, restore, and get the original weights back bit for bit."""
+    from types import SimpleNamespace
+
+    from arctictraining_amd import ArcticMoE
+    from arctictraining_amd.remap import (
+        detect_if_moe_model, remap_arctic_moe_to_orig_moe_mlp_params, remap_orig_moe_mlp_params_to_arctic_moe)
+
+    c, blk = _tiny_hf_block(dtype=torch.float32, E=8, K=2, H=64, I=32, seed=3)
+    c.architectures = ["Qwen3MoeForCausalLM"]
+    blk = blk.to(gpu_device)
+    E, I = c.num_experts, c.moe_intermediate_size
+    if as_list:  # the per-expert nn.Linear form the reference reads
+        fused, down = blk.experts.gate_up_proj.detach(), blk.experts.down_proj.detach()
+        experts = torch.nn.ModuleList()
+        for e in range(E):
+            ex = torch.nn.Module()
+            ex.gate_proj = torch.nn.Linear(c.hidden_size, I, bias=False, device=gpu_device)
+            ex.up_proj = torch.nn.Linear(c.hidden_size, I, bias=False, device=gpu_device)
+            ex.down_proj = torch.nn.Linear(I, c.hidden_size, bias=False, device=gpu_device)
+            with torch.no_grad():
+                ex.gate_proj.weight.copy_(fused[e, :I])
+                ex.up_proj.weight.copy_(fused[e, I:])
+                ex.down_proj.weight.copy_(down[e])
+            experts.append(ex)
+        mlp = torch.nn.Module()
+        mlp.gate, mlp.experts = blk.gate, experts
+    else:
+        mlp = blk
+    x = torch.randn(3, 17, c.hidden_size, device=gpu_device)
+    with torch.no_grad():
+        y_ref = blk(x)
+    saved = {k: v.detach().clone() for k, v in mlp.state_dict().items()}
+
+    layer = torch.nn.Module()
+    layer.mlp = mlp
+    dense_layer = torch.nn.Module()
+    dense_layer.mlp = torch.nn.Linear(4, 4)  # a layer without experts is left alone
+    model = torch.nn.Module()
+    model.model = torch.nn.Module()
+    model.model.layers = torch.nn.ModuleList([dense_layer, layer])
+    model.config, model.dtype = c, torch.float32
+    assert detect_if_moe_model(model)
+
+    remap_orig_moe_mlp_params_to_arctic_moe(model, ep_size=1, is_resume=False, device=gpu_device)
+    amoe = model.model.layers[1].mlp
+    assert isinstance(amoe, ArcticMoE) and isinstance(model.model.layers[0].mlp, torch.nn.Linear)
+    assert {n for n, _ in amoe.named_parameters()} == {"router_gate", "expert_gate_up", "expert_down"}
+    assert all(p.device.type == "meta" for p in amoe._hide["orig_mlp"].parameters())
+    with torch.no_grad():
+        y = amoe(x)
+    assert O.rel_l2(y.cpu(), y_ref.cpu()) <= 1e-5
+
+    remap_arctic_moe_to_orig_moe_mlp_params(model)
+    restored = model.model.layers[1].mlp
+    assert not isinstance(restored, ArcticMoE)
+    got = restored.state_dict()
+    assert got.keys() == saved.keys()
+    for k in saved:
+        assert torch.equal(got[k], saved[k]), k
