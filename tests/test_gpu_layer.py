@@ -208,3 +208,61 @@ def test_module_surface(gpu_device):
     layer(x)
     assert layer.timers.elapsed("amoe e2e") > 0 and layer.timers.elapsed("groupGeMM") > 0
     assert "expert_gate_up" in repr(layer)
+
+
+def test_layer_under_hip_graph_capture(gpu_device):
+    """Forward + backward captured into one HIP graph (nothing in the layer synchronises with the
+    host or allocates outside torch's capturable allocator): every replay, with eager work and
+    synchronisations between the replays, must reproduce the eager result bit for bit."""
+    dtype, T, H, E, K, I = torch.bfloat16, 1024, 256, 32, 4, 128
+    layer = build_layer(dtype, H, E, K, I, gpu_device)
+    g = torch.Generator().manual_seed(77)
+    with torch.no_grad():
+        for p in layer.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * 0.05).to(dtype))
+    xs = [torch.randn(T, H, generator=g).to(dtype).to(gpu_device) for _ in range(3)]
+    dys = [torch.randn(T, H, generator=g).to(dtype).to(gpu_device) for _ in range(3)]
+
+    def eager(x, dy):
+        for p in layer.parameters():
+            p.grad = None
+        xg = x.clone().requires_grad_(True)
+        y = layer(xg)
+        y.backward(dy)
+        return [y.detach().clone(), xg.grad.clone()] + [p.grad.clone() for p in layer.parameters()]
+
+    want = [eager(x, dy) for x, dy in zip(xs, dys)]
+
+    x_st = xs[0].clone().requires_grad_(True)
+    dy_st = dys[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):  # warm-up on the capture stream: allocator pools, cached offsets
+            for p in layer.parameters():
+                p.grad = None
+            x_st.grad = None
+            layer(x_st).backward(dy_st)
+    torch.cuda.current_stream().wait_stream(side)
+    for p in layer.parameters():
+        p.grad = None
+    x_st.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_st = layer(x_st)
+        y_st.backward(dy_st)
+    # the graph's outputs live in its private pool: keep them, the eager runs below rebind .grad
+    got = [y_st.detach(), x_st.grad] + [p.grad for p in layer.parameters()]
+    for r in (0, 1, 2, 1):
+        with torch.no_grad():
+            x_st.copy_(xs[r])
+            dy_st.copy_(dys[r])
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(got, want[r]):
+            assert torch.equal(a, b), f"replay of input {r} differs from the eager result"
+        # eager work between replays
+        _ = eager(xs[(r + 1) % 3], dys[(r + 1) % 3])
+        for p in layer.parameters():
+            p.grad = None
+        torch.cuda.synchronize()
