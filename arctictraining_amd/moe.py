@@ -94,24 +94,48 @@ class PhaseTimers:
 _SPLIT_OFFSETS = {}
 
 
-def _router_weight_grad(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
-    """dW_router [E,H] = d_logits^T [E,T] @ x [T,H] (autograd of moe.py:233).
-
-    The product is skinny (E rows) and deep (T): the library GEMM leaves most of the chip idle on
-    it.  For bf16 it is run as a split-K on the grouped weight-gradient kernel instead -- the
-    tokens are cut into chunks that play the role of experts, C[s] = d_logits[chunk s]^T @
-    x[chunk s] -- and the partial products are summed in float32."""
-    T, E = d_logits.shape
-    splits = 16
-    if x.dtype != torch.bfloat16 or E % 8 or T % (splits * 32):
-        return torch.matmul(d_logits.t(), x)
-    key = (T, splits, x.device)
+def _token_offsets(T: int, parts: int, device) -> torch.Tensor:
+    """int32 [parts + 1]: the T tokens cut into `parts` nearly equal consecutive chunks."""
+    key = (T, parts, device)
     offs = _SPLIT_OFFSETS.get(key)
     if offs is None:
-        offs = torch.arange(0, T + 1, T // splits, dtype=torch.int32, device=x.device)
+        offs = (torch.arange(parts + 1, dtype=torch.int64, device=device) * T // parts).to(torch.int32)
         _SPLIT_OFFSETS[key] = offs
-    part = ops.grouped_gemm_wgrad(d_logits, x, offs, splits, tile_cfg=1)  # [splits, E, H], 128x128 tiles
-    return part.sum(dim=0, dtype=torch.float32).to(x.dtype)
+    return offs
+
+
+def _token_ids(T: int, device) -> torch.Tensor:
+    key = (T, "ids", device)
+    ids = _SPLIT_OFFSETS.get(key)
+    if ids is None:
+        ids = torch.arange(T, dtype=torch.int32, device=device)
+        _SPLIT_OFFSETS[key] = ids
+    return ids
+
+
+def _dense_weight_grad(a: torch.Tensor, b: torch.Tensor, tile_cfg: int = 0, tile: int = 256) -> torch.Tensor:
+    """C [Kd,N] = a^T [Kd,T] @ b [T,N]: the weight gradient of a dense (not routed) linear map.
+
+    Few output tiles and a deep reduction over the tokens: run as a split-K on the grouped
+    weight-gradient kernel -- the tokens are cut into chunks that play the role of experts,
+    C[s] = a[chunk s]^T @ b[chunk s] -- and the partial products are summed in float32."""
+    T, Kd = a.shape
+    N = b.shape[1]
+    tiles = -(-Kd // tile) * -(-N // tile)
+    splits = max(1, min(16, 512 // tiles, T // 256)) if a.dtype == torch.bfloat16 else 1
+    part = ops.grouped_gemm_wgrad(a, b, _token_offsets(T, splits, a.device), splits, tile_cfg=tile_cfg)
+    if splits == 1:
+        return part[0]
+    return part.sum(dim=0, dtype=torch.float32).to(a.dtype)
+
+
+def _router_weight_grad(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """dW_router [E,H] = d_logits^T [E,T] @ x [T,H] (autograd of moe.py:233): skinny (E rows) and
+    deep (T), the library GEMM leaves most of the chip idle on it."""
+    T, E = d_logits.shape
+    if x.dtype != torch.bfloat16 or E % 8 or T < 16 * 32:
+        return torch.matmul(d_logits.t(), x)
+    return _dense_weight_grad(d_logits, x, tile_cfg=1, tile=128)  # 128x128 tiles
 
 
 class _ExpertLayerFn(torch.autograd.Function):
@@ -120,7 +144,7 @@ class _ExpertLayerFn(torch.autograd.Function):
     the load-balance hook :393-406)."""
 
     @staticmethod
-    def forward(ctx, x, router_gate, w_gate_up, w_down, replay, opts):
+    def forward(ctx, x, router_gate, w_gate_up, w_down, sh_gate_up, sh_down, sh_out_gate, replay, opts):
         T, H = x.shape
         E, K = opts["num_experts"], opts["top_k"]
         timers: PhaseTimers = opts["timers"]
@@ -144,14 +168,32 @@ class _ExpertLayerFn(torch.autograd.Function):
         out_s = ops.grouped_gemm_nn(inter_s, w_down, offsets, tile_cfg=cfg)
         timers.stop("groupGeMM")
 
+        # Shared expert (moe.py:305-314): a dense gated FFN over all T tokens, its output scaled per
+        # token by sigmoid(x @ w_out_gate).  It runs through the same kernels as one more expert that
+        # owns every token, the sigmoid in the role of the routing score; its output joins the
+        # combine as the addend of the per-token sum.
+        shared = sh_gate_up is not None
+        sh_gu = sh_inter_s = sh_sig = sh_out = None
+        if shared:
+            timers.start("shared-expert")
+            all_rows = _token_offsets(T, 1, x.device)
+            sh_sig = torch.sigmoid(torch.matmul(x, sh_out_gate)).float().reshape(T)
+            sh_gu, sh_inter_s = ops.grouped_gemm_gateup_act_fwd(
+                x, sh_gate_up.unsqueeze(0), all_rows, opts["act"], tile_cfg=cfg, row_scale=sh_sig
+            )
+            sh_out = ops.grouped_gemm_nn(sh_inter_s, sh_down.unsqueeze(0), all_rows, tile_cfg=cfg)
+            timers.stop("shared-expert")
+
         timers.start("moe-combine")
-        y = ops.combine_fwd(out_s, row_of, None)
+        # y[t] = sum_k out_s[row_of[t,k]] (+ the shared expert's row t)
+        y = ops.gather_rows_bwd(out_s, row_of, addend=sh_out) if shared else ops.combine_fwd(out_s, row_of, None)
         timers.stop("moe-combine")
 
         ctx.opts = opts
+        ctx.shared = shared
         ctx.save_for_backward(
             x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
-            gate_up, inter_s,
+            gate_up, inter_s, sh_gate_up, sh_down, sh_out_gate, sh_gu, sh_inter_s, sh_sig,
         )
         # scores in routed-row order, in the model dtype, as the reference returns them
         scores_out = scores_perm.to(x.dtype)
@@ -165,7 +207,7 @@ class _ExpertLayerFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy, _ds_perm):
         (x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
-         gate_up, inter_s) = ctx.saved_tensors
+         gate_up, inter_s, sh_gate_up, sh_down, sh_out_gate, sh_gu, sh_inter_s, sh_sig) = ctx.saved_tensors
         opts = ctx.opts
         E, K = opts["num_experts"], opts["top_k"]
         T = x.shape[0]
@@ -190,12 +232,33 @@ class _ExpertLayerFn(torch.autograd.Function):
             d_scores, probs, topk_idx, counts, x.dtype, opts["normalize"], opts["loss_coeff"] / T / opts["ep_size"]
         )
         d_router_gate = _router_weight_grad(d_logits, x) if ctx.needs_input_grad[1] else None
+
+        d_sh_gate_up = d_sh_down = d_sh_out_gate = d_sh_gu = d_pre = None
+        if ctx.shared:
+            # the same chain for the expert that owns every token; the "score" gradient comes
+            # back per token and goes on through the sigmoid
+            all_rows = _token_offsets(T, 1, x.device)
+            d_sh_inter_s = ops.grouped_gemm_nt(dy, sh_down.unsqueeze(0), all_rows, tile_cfg=cfg)
+            if ctx.needs_input_grad[5]:
+                d_sh_down = _dense_weight_grad(sh_inter_s, dy, tile_cfg=cfg)
+            d_sh_gu, d_sig = ops.gated_act_bwd(
+                sh_gu, d_sh_inter_s, opts["act"], row_scale=sh_sig, slot_of=_token_ids(T, x.device), tk=(T, 1)
+            )
+            if ctx.needs_input_grad[4]:
+                d_sh_gate_up = _dense_weight_grad(x, d_sh_gu, tile_cfg=cfg)
+            d_pre = (d_sig.reshape(T) * sh_sig * (1.0 - sh_sig)).to(x.dtype).unsqueeze(1)  # [T,1]
+            if ctx.needs_input_grad[6]:
+                d_sh_out_gate = torch.matmul(x.t(), d_pre)
+
         dx = None
         if ctx.needs_input_grad[0]:
             d_xp = ops.grouped_gemm_nt(d_gate_up, w_gate_up, offsets, tile_cfg=cfg)
-            dx_router = torch.matmul(d_logits, router_gate)
-            dx = ops.gather_rows_bwd(d_xp, row_of, addend=dx_router)
-        return dx, d_router_gate, d_w_gate_up, d_w_down, None, None
+            dx_dense = torch.matmul(d_logits, router_gate)
+            if ctx.shared:
+                dx_dense.addmm_(d_pre, sh_out_gate.t())
+                dx_dense += ops.grouped_gemm_nt(d_sh_gu, sh_gate_up.unsqueeze(0), all_rows, tile_cfg=cfg)
+            dx = ops.gather_rows_bwd(d_xp, row_of, addend=dx_dense)
+        return dx, d_router_gate, d_w_gate_up, d_w_down, d_sh_gate_up, d_sh_down, d_sh_out_gate, None, None
 
 
 class ArcticMoE(nn.Module):
@@ -285,19 +348,12 @@ class ArcticMoE(nn.Module):
             capture=self.capture,
         )
         replay = routing_replay_assignments if self.enable_routing_replay else None
-        output, scores = _ExpertLayerFn.apply(
-            x, self.router_gate, self.expert_gate_up, self.expert_down, replay, opts
-        )
+        shared = (None, None, None)
         if getattr(self._config, "use_shared_expert", False):
-            # dense shared expert with a sigmoid output gate (moe.py:305-314): library GEMMs
-            self.timers.start("shared-expert")
-            s_inter = torch.matmul(x, self.shared_expert_gate_up)
-            s_gate, s_up = s_inter[..., 0::2], s_inter[..., 1::2]
-            s_inter = s_up * self.act_fn(s_gate)
-            s_out = torch.matmul(s_inter, self.shared_expert_down)
-            s_out_gate = torch.matmul(x, self.shared_expert_output_gate)
-            output = output + s_out * torch.sigmoid(s_out_gate)
-            self.timers.stop("shared-expert")
+            shared = (self.shared_expert_gate_up, self.shared_expert_down, self.shared_expert_output_gate)
+        output, scores = _ExpertLayerFn.apply(
+            x, self.router_gate, self.expert_gate_up, self.expert_down, *shared, replay, opts
+        )
         output = output.reshape(orig_shape)
         self.timers.stop("amoe e2e")
         return (output, scores) if getattr(self._config, "return_router_scores", False) else output

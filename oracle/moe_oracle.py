@@ -21,6 +21,7 @@ reference tree):
   grouped GEMM         arctic_training/model/moe/moe.py:54-60
   gated expert FFN     arctic_training/model/moe/moe.py:176-193 (scale constants :110-111)
   weighted combine     arctic_training/model/moe/moe.py:450-461
+  shared expert        arctic_training/model/moe/moe.py:305-314 (parameters :116-130)
   weight layout        arctic_training/model/moe/utils.py:249-266
 
 Parity pins (all in tests/test_oracle_pins.py; the reference holds no golden
@@ -38,6 +39,9 @@ installed third-party HF block instead):
                         groups leave zero rows
   expert_ffn            de-interleaved chunk formulation; silu closed form
   combine               dense token-major sum
+  shared_expert         the installed transformers Qwen2MoeSparseMoeBlock
+                        (shared MLP + sigmoid gate) after weight-layout mapping,
+                        forward and all gradients; closed form on a 1x1 case
   load-balance hook     closed form d/dprobs of coeff * sum_e freq_e * mean_t p
   forward (autograd)    torch.autograd.gradcheck in fp64
   analytic_backward     equality with autograd of forward
@@ -241,6 +245,19 @@ def combine(moe_out: torch.Tensor, token_ids: torch.Tensor, scores_perm: torch.T
     return y.index_add(0, token_ids, moe_out * scores_perm[:, None])
 
 
+def shared_expert(x2d: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, w_out_gate: torch.Tensor, act: str):
+    """moe.py:305-314 -- a dense gated FFN every token goes through, scaled per token by a
+    sigmoid gate: (up * act(gate)) @ W_down * sigmoid(x @ w_out_gate).  w_gate_up [H, 2I] has the
+    gate in the even and the up projection in the odd columns, w_down is [I, H], w_out_gate [H, 1]."""
+    fn = activation(act)
+    s_inter = torch.matmul(x2d, w_gate_up)
+    s_gate, s_up = s_inter[..., 0::2], s_inter[..., 1::2]
+    s_inter = s_up * fn(s_gate)
+    s_out = torch.matmul(s_inter, w_down)
+    s_out_gate = torch.matmul(x2d, w_out_gate)
+    return s_out * torch.sigmoid(s_out_gate)
+
+
 # --------------------------------------------------------------------------
 # whole layer
 # --------------------------------------------------------------------------
@@ -256,8 +273,11 @@ def forward(
     logits_for_selection: Optional[torch.Tensor] = None,
     replay_assignments: Optional[torch.Tensor] = None,
     model_dtype: Optional[torch.dtype] = None,
+    shared=None,
 ) -> Dict[str, torch.Tensor]:
     """moe.py:219-323 on the default path at EP=1, differentiable with autograd.
+    `shared` = (shared_expert_gate_up, shared_expert_down, shared_expert_output_gate) adds the
+    shared expert (use_shared_expert=True).
 
     compute_dtype=None runs every op in the dtype of the inputs, with the
     reference's rounding after each op ("reference rounding" mode: what the
@@ -274,6 +294,8 @@ def forward(
         x2d, router_gate, expert_gate_up, expert_down = (
             t.to(compute_dtype) for t in (x2d, router_gate, expert_gate_up, expert_down)
         )
+        if shared is not None:
+            shared = tuple(t.to(compute_dtype) for t in shared)
         logits = router_linear(x2d, router_gate)
         # straight-through rounding of the logits to the model dtype
         logits = logits + (logits.detach().to(in_dtype).to(compute_dtype) - logits.detach())
@@ -301,6 +323,8 @@ def forward(
     cumsum = g["counts"].cumsum(0)
     gu, inter, out = expert_ffn(xp, expert_gate_up, expert_down, cumsum, cfg.act)
     y = combine(out, g["token_ids"], g["scores_perm"], cfg.top_k)
+    if shared is not None:
+        y = y + shared_expert(x2d, *shared, cfg.act)
     res = dict(g)
     res.update(logits=logits, xp=xp, gate_up=gu, inter=inter, moe_out=out, y=y.reshape(orig_shape), cumsum=cumsum)
     return res
@@ -314,10 +338,17 @@ def forward_backward(x, router_gate, expert_gate_up, expert_down, dy, cfg, **kw)
     leaves = [
         t.detach().to(leaf_dtype).clone().requires_grad_(True) for t in (x, router_gate, expert_gate_up, expert_down)
     ]
-    res = forward(*leaves, cfg, model_dtype=model_dtype, **kw)
+    shared = kw.pop("shared", None)
+    if shared is not None:
+        shared = tuple(t.detach().to(leaf_dtype).clone().requires_grad_(True) for t in shared)
+    res = forward(*leaves, cfg, model_dtype=model_dtype, shared=shared, **kw)
     y = res["y"]
     y.backward(dy.to(y.dtype).reshape(y.shape))
     res["dx"], res["d_router_gate"], res["d_expert_gate_up"], res["d_expert_down"] = (t.grad for t in leaves)
+    if shared is not None:
+        res["d_shared_expert_gate_up"], res["d_shared_expert_down"], res["d_shared_expert_output_gate"] = (
+            t.grad for t in shared
+        )
     return res
 
 

@@ -154,26 +154,43 @@ def test_layer_routing_replay_and_returned_scores(gpu_device):
         layer(x.to(gpu_device))
 
 
-def test_layer_shared_expert(gpu_device):
-    """Shared expert with a sigmoid output gate (moe.py:305-314) on top of the routed path."""
-    dtype, T, H, E, K, I = torch.float32, 128, 64, 4, 2, 32
+@pytest.mark.parametrize(
+    "dtype,T,H,E,K,I,act",
+    [
+        (torch.float32, 128, 64, 4, 2, 32, "silu"),
+        (torch.bfloat16, 1024, 256, 16, 4, 128, "silu"),
+        (torch.bfloat16, 2048 + 96, 512, 8, 2, 256, "gelu"),  # token count not a multiple of any tile
+    ],
+    ids=["fp32", "bf16", "bf16_ragged_gelu"],
+)
+def test_layer_shared_expert(gpu_device, dtype, T, H, E, K, I, act):
+    """Shared expert with a sigmoid output gate (moe.py:305-314) on top of the routed path:
+    output and every gradient, the shared expert's parameters included, against the oracle."""
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
     x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=10)
-    layer = build_layer(dtype, H, E, K, I, gpu_device, use_shared_expert=True)
+    layer = build_layer(dtype, H, E, K, I, gpu_device, use_shared_expert=True, act=getattr(F, act))
     g = torch.Generator().manual_seed(11)
-    sgu, sd, sg = (torch.randn(s, generator=g) * 0.05 for s in ((H, 2 * I), (I, H), (H, 1)))
+    sgu, sd, sg = ((torch.randn(s, generator=g) * 0.05).to(dtype) for s in ((H, 2 * I), (I, H), (H, 1)))
     with torch.no_grad():
         layer.shared_expert_gate_up.copy_(sgu)
         layer.shared_expert_down.copy_(sd)
         layer.shared_expert_output_gate.copy_(sg)
     got = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
-    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001)
-    ref = O.forward(x, wr, wgu, wd, ocfg, compute_dtype=torch.float64, logits_for_selection=got["cap"]["logits"])
-    x64 = x.double()
-    s_i = x64 @ sgu.double()
-    s_out = (s_i[:, 1::2] * F.silu(s_i[:, 0::2])) @ sd.double()
-    expect = ref["y"] + s_out * torch.sigmoid(x64 @ sg.double())
-    assert O.rel_l2(got["y"], expect) <= 1e-5
-    assert layer.shared_expert_down.grad is not None
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001, act=act)
+    ref = O.forward_backward(
+        x, wr, wgu, wd, dy, ocfg, compute_dtype=torch.float64, logits_for_selection=got["cap"]["logits"],
+        shared=(sgu, sd, sg),
+    )
+    assert torch.equal(got["cap"]["topk_idx"].long(), ref["topk_idx"])
+    for k in ("y", "dx", "d_router_gate", "d_expert_gate_up", "d_expert_down"):
+        assert O.rel_l2(got[k], ref[k]) <= tol, k
+    for name in ("shared_expert_gate_up", "shared_expert_down", "shared_expert_output_gate"):
+        grad = getattr(layer, name).grad
+        assert grad is not None and grad.shape == getattr(layer, name).shape
+        assert O.rel_l2(grad.cpu(), ref["d_" + name]) <= tol, name
+    # the shared expert must matter in this test: without it the output is far away
+    routed_only = O.forward(x, wr, wgu, wd, ocfg, compute_dtype=torch.float64, logits_for_selection=got["cap"]["logits"])
+    assert O.rel_l2(got["y"], routed_only["y"]) > 10 * tol
 
 
 def test_layer_is_deterministic(gpu_device):

@@ -300,6 +300,79 @@ def test_whole_layer_against_hf_block(norm):
     assert torch.allclose(ana["d_expert_gate_up"], dgu, atol=1e-12)
 
 
+def test_shared_expert_closed_form():
+    """H = I = 1: (x*wu) * silu(x*wg) * wd * sigmoid(x*wo), written out with math.exp."""
+    import math
+
+    x, wg, wu, wd, wo = 0.7, -1.3, 0.9, 1.7, 0.4
+    got = O.shared_expert(
+        torch.tensor([[x]], dtype=torch.float64),
+        torch.tensor([[wg, wu]], dtype=torch.float64),  # gate in the even, up in the odd column
+        torch.tensor([[wd]], dtype=torch.float64),
+        torch.tensor([[wo]], dtype=torch.float64),
+        "silu",
+    )
+    g = x * wg
+    want = (x * wu) * (g / (1 + math.exp(-g))) * wd / (1 + math.exp(-x * wo))
+    assert abs(float(got) - want) < 1e-15
+    # swapping the two interleaved columns must change the result (gate and up are not symmetric)
+    swapped = O.shared_expert(
+        torch.tensor([[x]], dtype=torch.float64), torch.tensor([[wu, wg]], dtype=torch.float64),
+        torch.tensor([[wd]], dtype=torch.float64), torch.tensor([[wo]], dtype=torch.float64), "silu",
+    )
+    assert abs(float(swapped) - want) > 1e-3
+
+
+def test_whole_layer_with_shared_expert_against_hf_block():
+    """The installed transformers Qwen2-MoE block = routed experts + shared MLP times a sigmoid
+    gate (the block the reference's shared-expert parameters are filled from, utils.py:268-289)."""
+    from transformers import Qwen2MoeConfig
+    from transformers.models.qwen2_moe.modeling_qwen2_moe import Qwen2MoeSparseMoeBlock
+
+    T, H, E, K, I = 24, 16, 6, 2, 12
+    c = Qwen2MoeConfig(
+        hidden_size=H, moe_intermediate_size=I, shared_expert_intermediate_size=I, intermediate_size=I, num_experts=E,
+        num_experts_per_tok=K, norm_topk_prob=True, hidden_act="silu", num_hidden_layers=1, num_attention_heads=1,
+        num_key_value_heads=1, vocab_size=8,
+    )
+    blk = Qwen2MoeSparseMoeBlock(c).to(torch.float64)
+    g = torch.Generator().manual_seed(21)
+    with torch.no_grad():
+        blk.gate.weight.copy_(torch.randn(E, H, generator=g, dtype=torch.float64) * 0.5)
+        blk.experts.gate_up_proj.copy_(torch.randn(E, 2 * I, H, generator=g, dtype=torch.float64) * 0.3)
+        blk.experts.down_proj.copy_(torch.randn(E, H, I, generator=g, dtype=torch.float64) * 0.3)
+        for lin in (blk.shared_expert.gate_proj, blk.shared_expert.up_proj, blk.shared_expert.down_proj, blk.shared_expert_gate):
+            lin.weight.copy_(torch.randn(lin.weight.shape, generator=g, dtype=torch.float64) * 0.3)
+    x = torch.randn(2, T // 2, H, generator=g, dtype=torch.float64)
+    dy = torch.randn(2, T // 2, H, generator=g, dtype=torch.float64)
+    xh = x.clone().requires_grad_(True)
+    yh = blk(xh)
+    yh.backward(dy)
+
+    gu = blk.experts.gate_up_proj.detach()
+    wgu = torch.stack((gu[:, :I, :].transpose(1, 2), gu[:, I:, :].transpose(1, 2)), dim=-1).reshape(E, H, 2 * I).contiguous()
+    wd = blk.experts.down_proj.detach().transpose(1, 2).contiguous()
+    sh = blk.shared_expert
+    # utils.py:272-289: nn.Linear weights transposed; gate / up interleaved on the last dimension
+    s_gu = torch.stack((sh.gate_proj.weight.detach().T, sh.up_proj.weight.detach().T), dim=-1).reshape(H, 2 * I).contiguous()
+    s_d = sh.down_proj.weight.detach().T.contiguous()
+    s_og = blk.shared_expert_gate.weight.detach().T.contiguous()
+    cfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, normalize_topk_scores=True, loss_coeff=0.0)
+    res = O.forward_backward(x, blk.gate.weight.detach(), wgu, wd, dy, cfg, shared=(s_gu, s_d, s_og))
+    # HF evaluates the router softmax in float32: agreement to float32 rounding downstream of it
+    assert torch.allclose(res["y"], yh.detach(), atol=5e-6)
+    assert torch.allclose(res["dx"], xh.grad, atol=5e-6)
+    assert torch.allclose(res["d_shared_expert_gate_up"][:, 0::2], sh.gate_proj.weight.grad.T, atol=1e-12)
+    assert torch.allclose(res["d_shared_expert_gate_up"][:, 1::2], sh.up_proj.weight.grad.T, atol=1e-12)
+    assert torch.allclose(res["d_shared_expert_down"], sh.down_proj.weight.grad.T, atol=1e-12)
+    assert torch.allclose(res["d_shared_expert_output_gate"], blk.shared_expert_gate.weight.grad.T, atol=1e-12)
+    # the shared expert's share of y is what is left when the routed layer is taken away
+    routed = O.forward(x, blk.gate.weight.detach(), wgu, wd, cfg)
+    assert torch.allclose(
+        res["y"].detach() - routed["y"], O.shared_expert(x.reshape(-1, H), s_gu, s_d, s_og, "silu").reshape(x.shape), atol=1e-12
+    )
+
+
 def test_reference_rounding_mode_close_to_exact():
     """bf16 with the reference's per-op rounding stays within the bf16 bar of
     the exact evaluation from the same rounded inputs."""

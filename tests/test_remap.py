@@ -204,3 +204,62 @@ def test_install_and_restore_hooks(gpu_device, as_list):
     assert got.keys() == saved.keys()
     for k in saved:
         assert torch.equal(got[k], saved[k]), k
+
+
+@pytest.mark.gpu
+def test_install_and_restore_hooks_shared_expert(gpu_device):
+    """The same round trip for a block with a shared expert and its sigmoid gate (the installed
+    transformers Qwen2-MoE block; utils.py:268-289 and :400-418)."""
+    from transformers import Qwen2MoeConfig
+    from transformers.models.qwen2_moe.modeling_qwen2_moe import Qwen2MoeSparseMoeBlock
+
+    from arctictraining_amd import ArcticMoE
+    from arctictraining_amd.remap import remap_arctic_moe_to_orig_moe_mlp_params, remap_orig_moe_mlp_params_to_arctic_moe
+
+    H, I, E, K = 64, 32, 8, 2
+    c = Qwen2MoeConfig(
+        hidden_size=H, moe_intermediate_size=I, shared_expert_intermediate_size=I, intermediate_size=I, num_experts=E,
+        num_experts_per_tok=K, norm_topk_prob=True, hidden_act="silu", num_hidden_layers=1, num_attention_heads=1,
+        num_key_value_heads=1, vocab_size=8,
+    )
+    c.architectures = ["Qwen2MoeForCausalLM"]
+    blk = Qwen2MoeSparseMoeBlock(c).to(torch.float32)
+    g = torch.Generator().manual_seed(5)
+    with torch.no_grad():
+        for p in blk.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.2)
+    blk = blk.to(gpu_device)
+    x = torch.randn(2, 19, H, generator=g).to(gpu_device)
+    xr = x.clone().requires_grad_(True)
+    y_ref = blk(xr)
+    y_ref.sum().backward()
+    saved = {k: v.detach().clone() for k, v in blk.state_dict().items()}
+    # gradients of the block's own run, in the block's layout (the install empties the block)
+    ref_grad = {k: p.grad.detach().cpu() for k, p in blk.named_parameters()}
+
+    layer = torch.nn.Module()
+    layer.mlp = blk
+    model = torch.nn.Module()
+    model.model = torch.nn.Module()
+    model.model.layers = torch.nn.ModuleList([layer])
+    model.config, model.dtype = c, torch.float32
+    remap_orig_moe_mlp_params_to_arctic_moe(model, device=gpu_device)
+    amoe = model.model.layers[0].mlp
+    assert isinstance(amoe, ArcticMoE) and amoe._config.use_shared_expert
+    amoe._config.loss_coeff = 0.0  # HF's block has no load-balance term in its gradient
+    xa = x.clone().requires_grad_(True)
+    y = amoe(xa)
+    y.sum().backward()
+    assert O.rel_l2(y.detach().cpu(), y_ref.detach().cpu()) <= 1e-5
+    assert O.rel_l2(xa.grad.cpu(), xr.grad.cpu()) <= 1e-5
+    assert O.rel_l2(amoe.shared_expert_gate_up.grad[:, 0::2].t().cpu(), ref_grad["shared_expert.gate_proj.weight"]) <= 1e-5
+    assert O.rel_l2(amoe.shared_expert_gate_up.grad[:, 1::2].t().cpu(), ref_grad["shared_expert.up_proj.weight"]) <= 1e-5
+    assert O.rel_l2(amoe.shared_expert_down.grad.t().cpu(), ref_grad["shared_expert.down_proj.weight"]) <= 1e-5
+    assert O.rel_l2(amoe.shared_expert_output_gate.grad.t().cpu(), ref_grad["shared_expert_gate.weight"]) <= 1e-5
+    assert O.rel_l2(amoe.router_gate.grad.cpu(), ref_grad["gate.weight"]) <= 1e-5
+
+    remap_arctic_moe_to_orig_moe_mlp_params(model)
+    got = model.model.layers[0].mlp.state_dict()
+    assert got.keys() == saved.keys()
+    for k in saved:
+        assert torch.equal(got[k], saved[k]), k
