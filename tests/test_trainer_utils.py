@@ -93,3 +93,74 @@ def test_timers_install_and_forward_breakdown():
     lines.clear()
     U.print_forward_breakdown(torch.nn.Linear(2, 2), printer=lines.append)
     assert lines == []
+
+
+class _FakeEngine:
+    """The attributes of a DeepSpeed engine the checkpoint routines read."""
+
+    def __init__(self, module, optimizer):
+        self.module, self.optimizer, self.lr_scheduler = module, optimizer, None
+        self.checkpoint_engine = U.TorchFileCheckpointEngine()
+        self.skipped_steps, self.global_steps, self.global_samples = 1, 7, 56
+        self.dp_world_size, self.mp_world_size, self.num_experts = 1, 1, [4]
+
+    def _get_ckpt_name(self, save_dir, tag):
+        return f"{save_dir}/{tag}/mp_rank_00_model_states.pt"
+
+    def _get_optimizer_ckpt_name(self, save_dir, tag, ep_rank):
+        return f"{save_dir}/{tag}/expp_rank_{ep_rank}_mp_rank_00_optim_states.pt"
+
+    def zero_optimization(self):
+        return False
+
+    def module_state_dict(self, exclude_frozen_parameters=False):
+        return self.module.state_dict()
+
+
+def test_checkpoint_files_round_trip(tmp_path):
+    torch.manual_seed(0)
+    m = _model()
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_(torch.randn_like(p))
+    opt = torch.optim.SGD(m.parameters(), lr=0.1, momentum=0.9)
+    eng = _FakeEngine(m, opt)
+    U.amoe_save_checkpoint(eng, str(tmp_path), "step7", client_state={"epoch": 3})
+    tag_dir = tmp_path / "step7"
+    assert sorted(p.name for p in tag_dir.iterdir()) == [
+        "ep_rank_0_moe_layer_0_model_states.pt", "ep_rank_0_moe_layer_1_model_states.pt",
+        "expp_rank_0_mp_rank_00_optim_states.pt", "mp_rank_00_model_states.pt",
+    ]
+    assert eng._curr_ckpt_path == str(tag_dir)
+    main = torch.load(tag_dir / "mp_rank_00_model_states.pt", weights_only=True)
+    assert main["global_steps"] == 7 and main["epoch"] == 3 and main["num_experts"] == [4]
+    # the main file holds the dense parameters only; each layer file holds that layer's ArcticMoE
+    assert set(main["module"]) == {"embed.weight", "layers.0.attn.weight", "layers.0.attn.bias",
+                                   "layers.1.attn.weight", "layers.1.attn.bias"}
+    layer1 = torch.load(tag_dir / "ep_rank_0_moe_layer_1_model_states.pt", weights_only=True)
+    assert set(layer1) == {"layers.1.mlp.router_gate", "layers.1.mlp.expert_gate_up", "layers.1.mlp.expert_down"}
+    # a file holds its own tensors only, not the storage they were views of
+    assert all(t.untyped_storage().nbytes() == t.numel() * t.element_size() for t in layer1.values())
+
+    fresh = _model()
+    state = dict(main["module"])
+    U.amoe_load_state_dict(str(tmp_path), "step7", state, old_moe_load=False, model=fresh, device="cpu")
+    assert set(state) == set(m.state_dict())
+    fresh.load_state_dict(state)
+    for (n, a), (_, b) in zip(m.named_parameters(), fresh.named_parameters()):
+        assert torch.equal(a, b), n
+
+
+def test_monkey_patch_needs_deepspeed():
+    import importlib.util
+
+    import pytest
+
+    if importlib.util.find_spec("deepspeed") is None:
+        with pytest.raises(ImportError, match="DeepSpeed"):
+            U.monkey_patch_ds_moe()
+    else:
+        U.monkey_patch_ds_moe()
+        from deepspeed.runtime.engine import DeepSpeedEngine
+
+        assert DeepSpeedEngine._save_moe_checkpoint is U.amoe_save_checkpoint
