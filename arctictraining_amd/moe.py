@@ -348,6 +348,12 @@ class ArcticMoE(nn.Module):
             capture=self.capture,
         )
         replay = routing_replay_assignments if self.enable_routing_replay else None
+        if x.shape[0] == 0:
+            # no tokens (the reference returns an empty tensor from the same code path): nothing to
+            # launch; the result still hangs off every parameter so that their gradients are zeros
+            output = (x + sum(p.sum() for p in self.parameters()) * 0).reshape(orig_shape)
+            self.timers.stop("amoe e2e")
+            return (output, x.new_zeros(0)) if getattr(self._config, "return_router_scores", False) else output
         shared = (None, None, None)
         if getattr(self._config, "use_shared_expert", False):
             shared = (self.shared_expert_gate_up, self.shared_expert_down, self.shared_expert_output_gate)

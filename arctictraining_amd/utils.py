@@ -134,7 +134,7 @@ def _saveable(engine, state):
     return _detached_copies(state) if engine.checkpoint_engine.preserves_storage_sharing() else state
 
 
-def amoe_save_checkpoint(self, save_dir, tag, client_state={}, exclude_frozen_parameters=False):
+def amoe_save_checkpoint(self, save_dir, tag, client_state=None, exclude_frozen_parameters=False):
     """Checkpoint of an engine whose model holds ArcticMoE layers (utils.py:546-630): one file per
     ArcticMoE layer and expert-parallel rank with that layer's whole state dict under its full
     module path, one optimizer file per expert-parallel rank, and -- from expert-parallel rank 0 --
@@ -182,7 +182,7 @@ def amoe_save_checkpoint(self, save_dir, tag, client_state={}, exclude_frozen_pa
         mp_world_size=self.mp_world_size,
         num_experts=self.num_experts,
     )
-    state.update(client_state)
+    state.update(client_state or {})
     self.checkpoint_engine.save(_saveable(self, state), save_path)
 
 

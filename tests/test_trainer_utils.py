@@ -164,3 +164,27 @@ def test_monkey_patch_needs_deepspeed():
         from deepspeed.runtime.engine import DeepSpeedEngine
 
         assert DeepSpeedEngine._save_moe_checkpoint is U.amoe_save_checkpoint
+
+
+def test_layer_with_no_tokens_returns_empty_and_zero_gradients():
+    """An empty batch launches nothing (so it runs without a GPU): empty output of the input's
+    shape, zero gradients for every parameter (what moe.py:219-323 yields for zero tokens)."""
+    m = _model(1).layers[0].mlp
+    with torch.no_grad():
+        for p in m.parameters():
+            p.fill_(0.5)
+    x = torch.zeros(2, 0, 16, requires_grad=True)
+    y = m(x)
+    assert y.shape == (2, 0, 16) and y.dtype == x.dtype
+    y.sum().backward()
+    for n, p in m.named_parameters():
+        assert p.grad is not None and not p.grad.any(), n
+
+
+def test_layer_needs_the_hip_library_for_real_work():
+    """There is no CPU fallback: tokens on a CPU tensor are refused, loudly."""
+    import pytest
+
+    m = _model(1).layers[0].mlp
+    with pytest.raises(RuntimeError):
+        m(torch.zeros(4, 16))
