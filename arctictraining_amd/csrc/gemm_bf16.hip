@@ -31,6 +31,7 @@
 // skew.
 #include "amoe_common.h"
 
+#include <atomic>
 #include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 mfma_bf16x8;
@@ -632,15 +633,19 @@ int launch_cfg(const GemmArgs& a, int grid, hipStream_t s)
 {
     auto kern = grouped_gemm_bf16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS>;
     constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
-    static bool attr_done = false;
-    if (!attr_done) {
+    // The LDS limit is an attribute of the kernel on one device: set once per device (bit d of the
+    // mask); setting it twice from racing threads is harmless.
+    static std::atomic<unsigned long long> attr_done{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;   // 63: never cached
+    if (dev == 63 || !(attr_done.load(std::memory_order_relaxed) >> dev & 1ull)) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (err != hipSuccess) {
             amoe_set_error("grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(err));
             return AMOE_ERR_LAUNCH;
         }
-        attr_done = true;
+        if (dev != 63) attr_done.fetch_or(1ull << dev, std::memory_order_relaxed);
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WGM * WGN * 64), lds_bytes, s, a);
     return amoe_check_launch("grouped_gemm_bf16");
