@@ -104,11 +104,38 @@ struct ElemTraits<bf16_t> {
     __device__ static __forceinline__ float round(float v) { return round_bf16(v); }
 };
 
+// Wave-wide reductions without LDS traffic: four DPP steps leave every lane of a 16-lane row
+// with the row's result (lanes exchanged inside quads, then between the quads of a half row,
+// then between the half rows), and the four rows are combined from one lane each.
+constexpr int AMOE_DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int AMOE_DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int AMOE_DPP_HALF_MIRROR = 0x141;  // row_half_mirror: lane i <- lane 7 - i of its half row
+constexpr int AMOE_DPP_MIRROR = 0x140;       // row_mirror: lane i <- lane 15 - i of its row
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t x)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xF, 0xF, true);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float x)
+{
+    return __uint_as_float(dpp_u32<CTRL>(__float_as_uint(x)));
+}
+
+__device__ __forceinline__ float row_lane_f32(float v, int lane)
+{
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), lane));
+}
+
 __device__ __forceinline__ float wave_sum(float v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, AMOE_WAVE);
-    return v;
+    v += dpp_f32<AMOE_DPP_QUAD_XOR1>(v);
+    v += dpp_f32<AMOE_DPP_QUAD_XOR2>(v);
+    v += dpp_f32<AMOE_DPP_HALF_MIRROR>(v);
+    v += dpp_f32<AMOE_DPP_MIRROR>(v);
+    return (row_lane_f32(v, 0) + row_lane_f32(v, 16)) + (row_lane_f32(v, 32) + row_lane_f32(v, 48));
 }
 
 // activations of the gated expert FFN (value and derivative)

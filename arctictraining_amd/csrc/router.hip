@@ -17,14 +17,32 @@ __device__ __forceinline__ unsigned long long sel_key(float v, int idx)
     return ((unsigned long long)u << 32) | (unsigned long long)(0xffffffffu - (uint32_t)idx);
 }
 
+template <int CTRL>
+__device__ __forceinline__ unsigned long long max_with_dpp(unsigned long long k)
+{
+    const uint32_t hi = (uint32_t)(k >> 32), lo = (uint32_t)k;
+    const unsigned long long other = ((unsigned long long)dpp_u32<CTRL>(hi) << 32) | dpp_u32<CTRL>(lo);
+    return other > k ? other : k;
+}
+
+__device__ __forceinline__ unsigned long long row_lane_u64(unsigned long long k, int lane)
+{
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(k >> 32), lane);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)k, lane);
+    return ((unsigned long long)hi << 32) | lo;
+}
+
+// wave-uniform maximum of the 64 keys
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        unsigned long long other = __shfl_xor(k, o, AMOE_WAVE);
-        k = other > k ? other : k;
-    }
-    return k;
+    k = max_with_dpp<AMOE_DPP_QUAD_XOR1>(k);
+    k = max_with_dpp<AMOE_DPP_QUAD_XOR2>(k);
+    k = max_with_dpp<AMOE_DPP_HALF_MIRROR>(k);
+    k = max_with_dpp<AMOE_DPP_MIRROR>(k);
+    const unsigned long long a = row_lane_u64(k, 0), b = row_lane_u64(k, 16);
+    const unsigned long long c = row_lane_u64(k, 32), d = row_lane_u64(k, 48);
+    const unsigned long long ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
 }
 
 template <typename T, int VPT>
@@ -66,7 +84,7 @@ router_topk_fwd_kernel(const T* __restrict__ logits, int n_tokens, int E, int K,
             }
         }
         // the owning lane broadcasts the logit
-        v_sel = __shfl(v_sel, e_sel & 63, AMOE_WAVE);
+        v_sel = row_lane_f32(v_sel, e_sel & 63);   // e_sel is wave-uniform
         if (k == 0) row_max = v_sel;
         if (lane == k) {
             top_v = v_sel;

@@ -8,6 +8,7 @@ reference, so the trainer's `layer.mlp = ArcticMoE(config)` (utils.py:320) works
 The whole routed-expert computation is one torch.autograd.Function whose forward and
 backward call the kernels stage by stage with no host synchronisation.
 """
+import contextlib
 import time
 from collections import defaultdict
 from dataclasses import dataclass
@@ -357,9 +358,11 @@ class ArcticMoE(nn.Module):
         shared = (None, None, None)
         if getattr(self._config, "use_shared_expert", False):
             shared = (self.shared_expert_gate_up, self.shared_expert_down, self.shared_expert_output_gate)
-        output, scores = _ExpertLayerFn.apply(
-            x, self.router_gate, self.expert_gate_up, self.expert_down, *shared, replay, opts
-        )
+        # the kernels are launched on the current device's current stream: make x's device current
+        with torch.cuda.device(x.device) if x.is_cuda else contextlib.nullcontext():
+            output, scores = _ExpertLayerFn.apply(
+                x, self.router_gate, self.expert_gate_up, self.expert_down, *shared, replay, opts
+            )
         output = output.reshape(orig_shape)
         self.timers.stop("amoe e2e")
         return (output, scores) if getattr(self._config, "return_router_scores", False) else output

@@ -24,6 +24,9 @@ def _dtype_code(t: torch.Tensor) -> int:
 def _chk(t: torch.Tensor, name: str, dtype=None) -> torch.Tensor:
     if not t.is_cuda:
         raise RuntimeError(f"{name} must live on the GPU (the HIP kernels have no CPU fallback)")
+    if t.device.index != torch.cuda.current_device():
+        # kernels are launched on the current device's current stream
+        raise RuntimeError(f"{name} lives on {t.device} but the current device is cuda:{torch.cuda.current_device()}")
     if not t.is_contiguous():
         raise RuntimeError(f"{name} must be contiguous")
     if dtype is not None and t.dtype != dtype:
