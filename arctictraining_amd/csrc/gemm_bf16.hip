@@ -292,21 +292,32 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             for (int q = 0; q < RPW_B; ++q)
                 dst[i][q] = scalar_load_i32(p.b_row_map + min(r0 + kt * BK + (wave * 64 + NT * i) / (BN / 8) + q, p.rows_total - 1));
     };
+    // Each fetched index passes through an empty asm statement as a scalar register first: a
+    // select between two values that are still loads from the index array would be folded into
+    // one load at a selected address, which turns the array into scratch memory.
     auto spread_a = [&](const int (&src)[PER_A][RPW_A], int (&dst)[PER_A]) {
 #pragma unroll
         for (int i = 0; i < PER_A; ++i) {
-            int v = src[i][0];
+            int v = 0;
 #pragma unroll
-            for (int q = 1; q < RPW_A; ++q) v = (lane / (BM / 8) == q) ? src[i][q] : v;
+            for (int q = 0; q < RPW_A; ++q) {
+                int sq = src[i][q];
+                asm("" : "+s"(sq));
+                v = (q == 0 || lane / (BM / 8) == q) ? sq : v;
+            }
             dst[i] = v;
         }
     };
     auto spread_b = [&](const int (&src)[PER_B][RPW_B], int (&dst)[PER_B]) {
 #pragma unroll
         for (int i = 0; i < PER_B; ++i) {
-            int v = src[i][0];
+            int v = 0;
 #pragma unroll
-            for (int q = 1; q < RPW_B; ++q) v = (lane / (BN / 8) == q) ? src[i][q] : v;
+            for (int q = 0; q < RPW_B; ++q) {
+                int sq = src[i][q];
+                asm("" : "+s"(sq));
+                v = (q == 0 || lane / (BN / 8) == q) ? sq : v;
+            }
             dst[i] = v;
         }
     };
