@@ -147,4 +147,9 @@ def test_transposing_reads_are_awaited_before_use(tmp_path):
         violations, n_tr = check_kernel(lines)
         total_tr += n_tr
         assert not violations, f"{name}: {violations[:5]}"
+        # No kernel may touch scratch (private) memory: neither spilled registers nor an index
+        # array the compiler could not keep in registers (a select between freshly loaded row
+        # indices once became a lookup in a scratch array and cost 5 % of the weight gradients).
+        private = [l.strip() for l in lines if re.match(r"\s*scratch_(load|store)", l)]
+        assert not private, f"{name} uses scratch memory: {private[:3]}"
     assert total_tr > 0, "no transposing reads found: the check is looking at the wrong instruction"
