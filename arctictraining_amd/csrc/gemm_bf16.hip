@@ -65,6 +65,7 @@ struct GemmArgs {
     int rows_total;  // weight gradient: length of the row maps
     int gm, gn;   // blocks of one XCD work on super-tiles of gm x gn tiles
     int sn;       // super-tiles along N
+    int max_mtiles;  // rows mode: entries of tile_map (those past the last tile hold expert -1)
 };
 
 enum { EPI_STORE = 0, EPI_GATED = 1 };
@@ -110,6 +111,9 @@ tile_map_kernel(const int32_t* __restrict__ offsets, int E, int bm, int4* __rest
         v.w = 0;
         tile_map[mt] = v;
     }
+    // entries past the last tile say so themselves: a workgroup learns that it has no tile from
+    // the entry it reads anyway, without first fetching the count
+    for (int mt = total + (int)threadIdx.x; mt < max_mtiles; mt += blockDim.x) tile_map[mt] = make_int4(-1, 0, 0, 0);
 }
 
 typedef short tr_i16x4 __attribute__((ext_vector_type(4)));
@@ -195,8 +199,9 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     int e, m0, mend, kt_count;
     int r0 = 0, r1 = 0;
     if (!WGRAD) {
-        if (pm >= *p.n_mtiles) return;
+        if (pm >= p.max_mtiles) return;
         int4 tm = p.tile_map[pm];
+        if (tm.x < 0) return;
         e = tm.x;
         m0 = tm.y;
         mend = tm.z;
@@ -483,8 +488,9 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             if (t < kt_count) {
                 if (A_MAP) spread_a(sa4[t], a_use);
                 if (B_MAP) spread_b(sb4[t], b_use);
-                dma_a(t, IC0{}, A_ALL{}, a_use);
+                // B first: its addresses are known, those of A may still wait for the row map
                 dma_b(t, IC0{}, B_ALL{}, b_use);
+                dma_a(t, IC0{}, A_ALL{}, a_use);
             }
         }
         if (kt_count > NSTAGE - 1) {
@@ -767,6 +773,7 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
     a.n_ntiles = (N + tc.bn - 1) / tc.bn;
     a.n_mt = 0;
     long long grid = 0;
+    a.max_mtiles = max_mtiles;
     rc = set_supertiles(a, max_mtiles, &grid);
     if (rc) return rc;
     return launch_any<true, B_KC, EPI, ACT>(a, tile_cfg, (int)grid, s);
