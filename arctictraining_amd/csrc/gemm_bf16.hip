@@ -153,6 +153,15 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
     __builtin_amdgcn_s_barrier();
 }
+// Activation for the bf16 epilogue: the sigmoid's division by the hardware reciprocal (1 ulp; the
+// result is rounded to bf16 next) instead of the ten-instruction IEEE division sequence.
+template <int ACT>
+__device__ __forceinline__ float act_fwd_fast(float g)
+{
+    if (ACT == AMOE_ACT_SILU) return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+    if (ACT == AMOE_ACT_GPT_OSS) return g * __builtin_amdgcn_rcpf(1.0f + __expf(-1.702f * g));
+    return act_fwd<ACT>(g);
+}
 using T_ = std::true_type;
 using F_ = std::false_type;
 
@@ -606,6 +615,15 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         constexpr bool full = decltype(FULL)::value;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
+            // gated: the scales of this lane's 8 rows of tile row i, fetched together ahead of
+            // the column loop (one wait for the batch instead of one per use)
+            float sc[4][2];
+            if (EPI == EPI_GATED) {
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4)
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) sc[v4][u] = s_rs[wm * WTM + i * 32 + 8 * v4 + 4 * lg + 2 * u + odd1];
+            }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const bool col_ok = full || (n0 + wn * WTN + j * 32 + (lj & ~1) < p.N);
@@ -621,7 +639,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
                         const uint32_t pk = __builtin_amdgcn_perm(got, own, swap_sel);
                         const bool ok = full || (col_ok && m0 + rt + 2 * u + odd1 < mend);
                         if (EPI == EPI_GATED)
-                            h[u] = s_rs[rt + 2 * u + odd1] * bf16_hi(pk) * act_fwd<ACT>(bf16_lo(pk));
+                            h[u] = sc[v >> 2][u] * bf16_hi(pk) * act_fwd_fast<ACT>(bf16_lo(pk));
                         if (want_c && ok) {
                             char* rowp = cbase + ((long long)(rq + 2 * u) * p.ldc + j * 32) * 2;
                             *reinterpret_cast<uint32_t*>(rowp + loff) = pk;
