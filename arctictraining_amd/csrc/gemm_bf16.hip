@@ -210,6 +210,9 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     if (!WGRAD) {
         if (pm >= p.max_mtiles) return;
         int4 tm = p.tile_map[pm];
+        // the whole entry in one load (pinned here; otherwise .y and .z are fetched by a second,
+        // dependent load behind the test of .x)
+        asm volatile("" : "+s"(tm.x), "+s"(tm.y), "+s"(tm.z));
         if (tm.x < 0) return;
         e = tm.x;
         m0 = tm.y;
