@@ -22,6 +22,8 @@ CONFIGS = {
     "c5_stress_scaled": (torch.bfloat16, 4096, 256, 64, 4, 192, dict(bias_hot=0.55, n_hot=4, n_dead=8)),
     "tiny_fp32": (torch.float32, 37, 64, 5, 3, 32, {}),
     "tiny_bf16_k1": (torch.bfloat16, 130, 64, 4, 1, 64, {}),
+    # the largest expert count and top-k the kernels take; most experts get a handful of rows, some none
+    "widest_routing": (torch.bfloat16, 300, 128, 512, 16, 64, {}),
 }
 
 
