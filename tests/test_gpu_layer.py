@@ -285,3 +285,36 @@ def test_layer_under_hip_graph_capture(gpu_device):
         for p in layer.parameters():
             p.grad = None
         torch.cuda.synchronize()
+
+
+def test_layer_with_frozen_parameters_and_plain_inference(gpu_device):
+    """Gradients are only produced for what asks for them: frozen expert weights and a frozen
+    router get none, the rest equal a run in which everything is trainable; a forward under
+    no_grad gives the same output."""
+    dtype, T, H, E, K, I = torch.bfloat16, 512, 128, 8, 2, 64
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=21)
+    layer = build_layer(dtype, H, E, K, I, gpu_device)
+    full = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+
+    layer.expert_gate_up.requires_grad_(False)
+    layer.router_gate.requires_grad_(False)
+    for p in layer.parameters():
+        p.grad = None
+    xg = x.to(gpu_device).requires_grad_(True)
+    y = layer(xg)
+    y.backward(dy.to(gpu_device))
+    assert layer.expert_gate_up.grad is None and layer.router_gate.grad is None
+    assert torch.equal(y.detach().cpu(), full["y"])
+    assert torch.equal(xg.grad.cpu(), full["dx"])
+    assert torch.equal(layer.expert_down.grad.cpu(), full["d_expert_down"])
+
+    # input that needs no gradient: only the parameter gradients are computed
+    layer.expert_gate_up.requires_grad_(True)
+    for p in layer.parameters():
+        p.grad = None
+    layer(x.to(gpu_device)).backward(dy.to(gpu_device))
+    assert torch.equal(layer.expert_gate_up.grad.cpu(), full["d_expert_gate_up"])
+
+    with torch.no_grad():
+        y2 = layer(x.to(gpu_device))
+    assert not y2.requires_grad and torch.equal(y2.cpu(), full["y"])
