@@ -44,7 +44,9 @@ int check_gemm_common(const char* what, int dtype, int R, int E, int d0, int d1,
     AMOE_REQUIRE(R > 0 && E > 0 && d0 > 0 && d1 > 0, AMOE_ERR_BAD_ARG, "%s: sizes must be positive (R=%d E=%d %d %d)",
                  what, R, E, d0, d1);
     AMOE_REQUIRE(E <= AMOE_MAX_EXPERTS, AMOE_ERR_UNSUPPORTED, "%s: E=%d exceeds %d", what, E, AMOE_MAX_EXPERTS);
-    AMOE_REQUIRE(tile_cfg >= 0 && tile_cfg <= 5 && tile_cfg != 4, AMOE_ERR_BAD_ARG, "%s: tile_cfg %d is not one of 0, 1, 2, 3, 5", what, tile_cfg);
+    const int shape = tile_cfg & ~AMOE_TILE_MAP_READY;
+    AMOE_REQUIRE(tile_cfg >= 0 && shape <= 5 && shape != 4, AMOE_ERR_BAD_ARG,
+                 "%s: tile_cfg %d is not one of 0, 1, 2, 3, 5 (optionally | AMOE_TILE_MAP_READY)", what, tile_cfg);
     AMOE_REQUIRE((long long)R * d0 < (1ll << 32) && (long long)R * d1 < (1ll << 32) && (long long)d0 * d1 < (1ll << 32),
                  AMOE_ERR_UNSUPPORTED, "%s: an operand exceeds 2^32 elements", what);
     return AMOE_OK;

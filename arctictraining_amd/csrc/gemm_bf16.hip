@@ -748,17 +748,19 @@ AMOE_EXPORT size_t amoe_grouped_gemm_workspace_bytes(int R, int E)
     return 16 + sizeof(int4) * (size_t)ws_max_mtiles(R, E, 64);
 }
 
+// ready: the workspace already holds the map for these arguments (AMOE_TILE_MAP_READY); nothing is launched
 int amoe_build_tile_map(const int32_t* offsets, int R, int E, int bm, void* workspace, size_t workspace_bytes,
-                        const int4** tile_map, const int32_t** n_mtiles, int* max_mtiles, hipStream_t s)
+                        const int4** tile_map, const int32_t** n_mtiles, int* max_mtiles, hipStream_t s, bool ready)
 {
     AMOE_REQUIRE(workspace_bytes >= amoe_grouped_gemm_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
                  "grouped_gemm: workspace %zu < %zu bytes", workspace_bytes, amoe_grouped_gemm_workspace_bytes(R, E));
     int32_t* cnt = (int32_t*)workspace;
     int4* map = (int4*)((char*)workspace + 16);
     *max_mtiles = ws_max_mtiles(R, E, bm);
-    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(512), 0, s, offsets, E, bm, map, cnt, *max_mtiles);
     *tile_map = map;
     *n_mtiles = cnt;
+    if (ready) return AMOE_OK;
+    hipLaunchKernelGGL(tile_map_kernel, dim3(1), dim3(512), 0, s, offsets, E, bm, map, cnt, *max_mtiles);
     return amoe_check_launch("tile_map");
 }
 
@@ -768,11 +770,13 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
                          void* C2, const float* row_scale, int R, int E, int Kred, int N, int ldb, long long strideB, void* workspace,
                          size_t workspace_bytes, int tile_cfg, hipStream_t s)
 {
+    const bool map_ready = (tile_cfg & AMOE_TILE_MAP_READY) != 0;
+    tile_cfg &= ~AMOE_TILE_MAP_READY;
     TileCfg tc = pick_cfg(tile_cfg);
     GemmArgs a = {};
     int max_mtiles = 0;
     int rc = amoe_build_tile_map(offsets, R, E, tc.bm, workspace, workspace_bytes, &a.tile_map, &a.n_mtiles,
-                                 &max_mtiles, s);
+                                 &max_mtiles, s, map_ready);
     if (rc) return rc;
     a.A = (const bf16_t*)A;
     a.B = (const bf16_t*)B;
@@ -828,6 +832,7 @@ int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const i
 int amoe_bf16_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
                     const int32_t* offsets, void* C, int R, int E, int Kd, int N, int tile_cfg, hipStream_t s)
 {
+    tile_cfg &= ~AMOE_TILE_MAP_READY;   // no tile map in the weight gradient
     TileCfg tc = pick_cfg(tile_cfg);
     GemmArgs a = {};
     a.A = (const bf16_t*)A;

@@ -8,7 +8,7 @@
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float mfma_f32x16;
 
 int amoe_build_tile_map(const int32_t* offsets, int R, int E, int bm, void* workspace, size_t workspace_bytes,
-                        const int4** tile_map, const int32_t** n_mtiles, int* max_mtiles, hipStream_t s);
+                        const int4** tile_map, const int32_t** n_mtiles, int* max_mtiles, hipStream_t s, bool ready);
 
 namespace {
 
@@ -159,7 +159,8 @@ int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const 
 {
     GemmArgsF32 a = {};
     int max_mtiles = 0;
-    int rc = amoe_build_tile_map(offsets, R, E, BM, workspace, workspace_bytes, &a.tile_map, &a.n_mtiles, &max_mtiles, s);
+    int rc = amoe_build_tile_map(offsets, R, E, BM, workspace, workspace_bytes, &a.tile_map, &a.n_mtiles, &max_mtiles, s,
+                                 /*ready=*/false);
     if (rc) return rc;
     a.A = (const float*)A;
     a.B = (const float*)B;

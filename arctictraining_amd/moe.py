@@ -163,10 +163,13 @@ class _ExpertLayerFn(torch.autograd.Function):
         # (s * inter) @ W_down == s * (inter @ W_down), and the combine becomes a plain sum.
         timers.start("groupGeMM")
         cfg = opts["tile_cfg"]
+        # the four row-grouped GEMMs of a step share one tile map: built once here, kept for backward
+        ws = ops.gemm_workspace(T * K, E, x.device)
         gate_up, inter_s = ops.grouped_gemm_gateup_act_fwd(
-            x, w_gate_up, offsets, opts["act"], a_row_map=token_of, n_rows=T * K, tile_cfg=cfg, row_scale=scores_perm
+            x, w_gate_up, offsets, opts["act"], a_row_map=token_of, n_rows=T * K, tile_cfg=cfg, row_scale=scores_perm,
+            workspace=ws,
         )
-        out_s = ops.grouped_gemm_nn(inter_s, w_down, offsets, tile_cfg=cfg)
+        out_s = ops.grouped_gemm_nn(inter_s, w_down, offsets, tile_cfg=cfg, workspace=ws, map_ready=True)
         timers.stop("groupGeMM")
 
         # Shared expert (moe.py:305-314): a dense gated FFN over all T tokens, its output scaled per
@@ -192,13 +195,16 @@ class _ExpertLayerFn(torch.autograd.Function):
 
         ctx.opts = opts
         ctx.shared = shared
+        ctx.gemm_ws = ws
         ctx.save_for_backward(
             x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
             gate_up, inter_s, sh_gate_up, sh_down, sh_out_gate, sh_gu, sh_inter_s, sh_sig,
         )
         # scores in routed-row order, in the model dtype, as the reference returns them
-        scores_out = scores_perm.to(x.dtype)
+        # (only when the caller returns them: return_router_scores)
+        scores_out = scores_perm.to(x.dtype) if opts["want_scores"] else scores_perm.new_empty(0)
         ctx.mark_non_differentiable(scores_out)
+        ctx.set_materialize_grads(False)  # no zero-filled gradient for the scores output
         cap = opts.get("capture")
         if cap is not None:
             cap.update(logits=logits, probs=probs, topk_idx=topk_idx, scores=scores, counts=counts, offsets=offsets,
@@ -214,10 +220,14 @@ class _ExpertLayerFn(torch.autograd.Function):
         T = x.shape[0]
         R = T * K
         cfg = opts["tile_cfg"]
+        if dy is None:  # the output took no part in the loss
+            return (None,) * 9
         dy = dy.contiguous()
 
         # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMMs' loads
-        d_inter_s = ops.grouped_gemm_nt(dy, w_down, offsets, a_row_map=token_of, n_rows=R, tile_cfg=cfg)
+        ws = ctx.gemm_ws  # still holds the forward's tile map
+        d_inter_s = ops.grouped_gemm_nt(dy, w_down, offsets, a_row_map=token_of, n_rows=R, tile_cfg=cfg, workspace=ws,
+                                        map_ready=True)
         d_w_down = None
         if ctx.needs_input_grad[3]:
             d_w_down = ops.grouped_gemm_wgrad(inter_s, dy, offsets, E, tile_cfg=cfg, b_row_map=token_of)
@@ -253,7 +263,7 @@ class _ExpertLayerFn(torch.autograd.Function):
 
         dx = None
         if ctx.needs_input_grad[0]:
-            d_xp = ops.grouped_gemm_nt(d_gate_up, w_gate_up, offsets, tile_cfg=cfg)
+            d_xp = ops.grouped_gemm_nt(d_gate_up, w_gate_up, offsets, tile_cfg=cfg, workspace=ws, map_ready=True)
             dx_dense = torch.matmul(d_logits, router_gate)
             if ctx.shared:
                 dx_dense.addmm_(d_pre, sh_out_gate.t())
@@ -345,6 +355,7 @@ class ArcticMoE(nn.Module):
             ep_size=self.ep_size,
             act=self._act_code,
             tile_cfg=self.tile_cfg,
+            want_scores=bool(getattr(self._config, "return_router_scores", False)),
             timers=self.timers,
             capture=self.capture,
         )

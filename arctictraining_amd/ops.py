@@ -11,6 +11,7 @@ from . import _lib
 
 F32, BF16 = 0, 1
 ACT_SILU, ACT_GELU, ACT_RELU, ACT_GPT_OSS = 0, 1, 2, 3
+TILE_MAP_READY = 0x100  # AMOE_TILE_MAP_READY
 
 
 def _dtype_code(t: torch.Tensor) -> int:
@@ -163,9 +164,20 @@ def combine_bwd(dy, moe_out, row_of, scores, need_d_out: bool = True) -> Tuple[O
     return d_out, d_scores
 
 
-def _gemm_workspace(R: int, E: int, device) -> torch.Tensor:
+def gemm_workspace(R: int, E: int, device) -> torch.Tensor:
+    """Workspace of the row-grouped GEMMs (holds the tile map built from `offsets`).  Calls that
+    share R, E, offsets, dtype and tile shape may share one workspace; all but the first can then
+    pass map_ready=True and skip rebuilding the map."""
     n = _lib.load().amoe_grouped_gemm_workspace_bytes(R, E)
     return torch.empty(max(n, 16), dtype=torch.uint8, device=device)
+
+
+def _ws_and_cfg(R, E, device, tile_cfg, workspace, map_ready):
+    if workspace is None:
+        if map_ready:
+            raise RuntimeError("map_ready needs the workspace that holds the map")
+        workspace = gemm_workspace(R, E, device)
+    return workspace, (tile_cfg | TILE_MAP_READY) if map_ready else tile_cfg
 
 
 def grouped_gemm_gateup_act_fwd(
@@ -178,6 +190,8 @@ def grouped_gemm_gateup_act_fwd(
     tile_cfg: int = 0,
     want_gate_up: bool = True,
     row_scale: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None,
+    map_ready: bool = False,
 ):
     """gate_up [R,2I], inter [R,I] (times row_scale [R] when given) from xp [R,H] (or x [T,H] with
     a_row_map [R]) and w [E,H,2I]."""
@@ -194,7 +208,7 @@ def grouped_gemm_gateup_act_fwd(
     I = I2 // 2
     gate_up = torch.empty((R, I2), dtype=xp.dtype, device=xp.device) if want_gate_up else None
     inter = torch.empty((R, I), dtype=xp.dtype, device=xp.device)
-    ws = _gemm_workspace(R, E, xp.device)
+    ws, tile_cfg = _ws_and_cfg(R, E, xp.device, tile_cfg, workspace, map_ready)
     rc = lib.amoe_grouped_gemm_gateup_act_fwd(
         xp.data_ptr(), _ptr(a_row_map), w_gate_up.data_ptr(), offsets.data_ptr(), _ptr(row_scale), _ptr(gate_up),
         inter.data_ptr(),
@@ -204,7 +218,8 @@ def grouped_gemm_gateup_act_fwd(
     return gate_up, inter
 
 
-def grouped_gemm_nn(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 0) -> torch.Tensor:
+def grouped_gemm_nn(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 0, workspace=None,
+                    map_ready: bool = False) -> torch.Tensor:
     """C[rows_e,:] = A[rows_e,:] @ B[e];  A [R,Kd], B [E,Kd,N] -> C [R,N]."""
     lib = _lib.load()
     _chk(A, "A")
@@ -213,7 +228,7 @@ def grouped_gemm_nn(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 
     E, Kd, N = B.shape
     R = int(n_rows if n_rows is not None else (a_row_map.numel() if a_row_map is not None else A.shape[0]))
     C = torch.empty((R, N), dtype=A.dtype, device=A.device)
-    ws = _gemm_workspace(R, E, A.device)
+    ws, tile_cfg = _ws_and_cfg(R, E, A.device, tile_cfg, workspace, map_ready)
     rc = lib.amoe_grouped_gemm_nn(
         A.data_ptr(), _ptr(a_row_map), B.data_ptr(), offsets.data_ptr(), C.data_ptr(), _dtype_code(A), R, E, Kd, N,
         ws.data_ptr(), ws.numel(), tile_cfg, _stream()
@@ -222,7 +237,8 @@ def grouped_gemm_nn(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 
     return C
 
 
-def grouped_gemm_nt(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 0) -> torch.Tensor:
+def grouped_gemm_nt(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 0, workspace=None,
+                    map_ready: bool = False) -> torch.Tensor:
     """C[rows_e,:] = A[rows_e,:] @ B[e]^T;  A [R,N], B [E,Kd,N] -> C [R,Kd]."""
     lib = _lib.load()
     _chk(A, "A")
@@ -231,7 +247,7 @@ def grouped_gemm_nt(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 
     E, Kd, N = B.shape
     R = int(n_rows if n_rows is not None else (a_row_map.numel() if a_row_map is not None else A.shape[0]))
     C = torch.empty((R, Kd), dtype=A.dtype, device=A.device)
-    ws = _gemm_workspace(R, E, A.device)
+    ws, tile_cfg = _ws_and_cfg(R, E, A.device, tile_cfg, workspace, map_ready)
     rc = lib.amoe_grouped_gemm_nt(
         A.data_ptr(), _ptr(a_row_map), B.data_ptr(), offsets.data_ptr(), C.data_ptr(), _dtype_code(A), R, E, Kd, N,
         ws.data_ptr(), ws.numel(), tile_cfg, _stream()

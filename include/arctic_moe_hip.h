@@ -123,6 +123,14 @@ int amoe_combine_bwd(const void* dy, const void* moe_out, const int32_t* row_of,
 size_t amoe_grouped_gemm_workspace_bytes(int R, int E);
 
 /*
+ * May be OR-ed into `tile_cfg` of the three row-grouped GEMMs below: the workspace passed in
+ * still holds the tile map that an earlier row-grouped call built from the same offsets, R, E,
+ * dtype and tile shape, and nobody has written to it since; the map is then not built again
+ * (the forward and backward GEMMs of one layer step all use the same map).
+ */
+#define AMOE_TILE_MAP_READY 0x100
+
+/*
  * Grouped gate_up GEMM with the gated activation fused (moe.py:54-60 + 187-191):
  *   gate_up[rows_e, :] = xp[rows_e, :] @ w_gate_up[e]                          [R,2I]
  *   inter[r, i] = row_scale[r] * gate_up[r, 2i+1] * act(gate_up[r, 2i])        [R,I]

@@ -99,6 +99,8 @@ def test_gemm_argument_errors(lib):
     assert lib.amoe_grouped_gemm_wgrad(P, None, P, None, P, P, 0, 128, 1000, 64, 64, 0, None) == -2  # E too large
     assert lib.amoe_grouped_gemm_wgrad(P, P, P, P, P, P, 1, 128, 4, 64, 64, 0, None) == -2  # both operands gathered
     assert lib.amoe_grouped_gemm_nn(P, None, P, P, P, 1, 128, 4, 64, 64, P, big, 4, None) == -1  # retired tile_cfg
+    assert lib.amoe_grouped_gemm_nn(P, None, P, P, P, 1, 128, 4, 64, 64, P, big, 0x100 | 4, None) == -1  # flag on a bad shape
+    assert lib.amoe_grouped_gemm_nn(P, None, P, P, P, 1, 128, 4, 64, 64, P, big, 0x200, None) == -1  # unknown flag
     assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, None, P, P, 1, 128, 4, 64, 64, 7, P, big, 0, None) == -1
     assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, None, None, P, 0, 128, 4, 64, 64, 0, P, big, 0, None) == -2
 

@@ -393,3 +393,25 @@ def test_grouped_gemm_rows_outside_groups_untouched(ops, gpu_device):
     C = lib_ops.grouped_gemm_nn(A, B, offs)
     ref = O.grouped_gemm(A.cpu().double()[:440], B.cpu().double(), counts.cumsum(0))
     assert O.rel_l2(C[:440].cpu(), ref) <= 4e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_grouped_gemm_shared_tile_map(ops, gpu_device, dtype):
+    """Row-grouped GEMMs over the same offsets may share one workspace: calls after the first pass
+    map_ready (AMOE_TILE_MAP_READY) and reuse the tile map it holds; results are unchanged."""
+    g = torch.Generator().manual_seed(9)
+    R, E, Kd, N = 1500, 6, 96, 160
+    counts = torch.tensor([300, 0, 517, 255, 1, 427])
+    offs = _offsets(counts, gpu_device)
+    A = torch.randn(R, Kd, generator=g).to(dtype).to(gpu_device)
+    A2 = torch.randn(R, N, generator=g).to(dtype).to(gpu_device)
+    B = (torch.randn(E, Kd, N, generator=g) * 0.1).to(dtype).to(gpu_device)
+    ws = ops.gemm_workspace(R, E, gpu_device)
+    c_first = ops.grouped_gemm_nn(A, B, offs, workspace=ws)                      # builds the map
+    c_again = ops.grouped_gemm_nn(A, B, offs, workspace=ws, map_ready=True)      # reuses it
+    d_again = ops.grouped_gemm_nt(A2, B, offs, workspace=ws, map_ready=True)
+    assert torch.equal(c_first, ops.grouped_gemm_nn(A, B, offs))
+    assert torch.equal(c_again, c_first)
+    assert torch.equal(d_again, ops.grouped_gemm_nt(A2, B, offs))
+    with pytest.raises(RuntimeError, match="workspace"):
+        ops.grouped_gemm_nn(A, B, offs, map_ready=True)
