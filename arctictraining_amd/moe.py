@@ -10,7 +10,7 @@ backward call the kernels stage by stage with no host synchronisation.
 """
 import contextlib
 import time
-from collections import defaultdict
+from collections import OrderedDict, defaultdict
 from dataclasses import dataclass
 from typing import Any, Optional
 
@@ -92,26 +92,46 @@ class PhaseTimers:
         return self.times[name]
 
 
-_SPLIT_OFFSETS = {}
+class _SmallTensorCache:
+    """A few small index tensors keyed by (size, kind, device), least recently used evicted first:
+    the token count changes from step to step with packed variable-length batches, so the cache
+    must not grow with the number of distinct sizes seen.  Nothing is stored while a HIP graph is
+    being captured (a tensor created there lives in the graph's private pool and only holds its
+    values after a replay)."""
+
+    def __init__(self, max_entries: int = 8):
+        self.max_entries = max_entries
+        self._d = OrderedDict()
+
+    def get(self, key, make):
+        t = self._d.get(key)
+        if t is not None:
+            self._d.move_to_end(key)
+            return t
+        t = make()
+        if not (t.is_cuda and torch.cuda.is_current_stream_capturing()):
+            self._d[key] = t
+            while len(self._d) > self.max_entries:
+                self._d.popitem(last=False)
+        return t
+
+    def __len__(self):
+        return len(self._d)
+
+
+_INDEX_CACHE = _SmallTensorCache()
 
 
 def _token_offsets(T: int, parts: int, device) -> torch.Tensor:
     """int32 [parts + 1]: the T tokens cut into `parts` nearly equal consecutive chunks."""
-    key = (T, parts, device)
-    offs = _SPLIT_OFFSETS.get(key)
-    if offs is None:
-        offs = (torch.arange(parts + 1, dtype=torch.int64, device=device) * T // parts).to(torch.int32)
-        _SPLIT_OFFSETS[key] = offs
-    return offs
+    return _INDEX_CACHE.get(
+        (T, parts, str(device)),
+        lambda: (torch.arange(parts + 1, dtype=torch.int64, device=device) * T // parts).to(torch.int32),
+    )
 
 
 def _token_ids(T: int, device) -> torch.Tensor:
-    key = (T, "ids", device)
-    ids = _SPLIT_OFFSETS.get(key)
-    if ids is None:
-        ids = torch.arange(T, dtype=torch.int32, device=device)
-        _SPLIT_OFFSETS[key] = ids
-    return ids
+    return _INDEX_CACHE.get((T, "ids", str(device)), lambda: torch.arange(T, dtype=torch.int32, device=device))
 
 
 def _dense_weight_grad(a: torch.Tensor, b: torch.Tensor, tile_cfg: int = 0, tile: int = 256) -> torch.Tensor:
@@ -200,11 +220,14 @@ class _ExpertLayerFn(torch.autograd.Function):
             x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
             gate_up, inter_s, sh_gate_up, sh_down, sh_out_gate, sh_gu, sh_inter_s, sh_sig,
         )
-        # scores in routed-row order, in the model dtype, as the reference returns them
-        # (only when the caller returns them: return_router_scores)
-        scores_out = scores_perm.to(x.dtype) if opts["want_scores"] else scores_perm.new_empty(0)
-        ctx.mark_non_differentiable(scores_out)
-        ctx.set_materialize_grads(False)  # no zero-filled gradient for the scores output
+        # scores in routed-row order, in the model dtype, as the reference returns them (moe.py:323,
+        # only when return_router_scores); they stay attached to the graph like the reference's
+        if opts["want_scores"]:
+            scores_out = scores_perm.to(x.dtype)
+        else:
+            scores_out = scores_perm.new_empty(0)
+            ctx.mark_non_differentiable(scores_out)
+        ctx.set_materialize_grads(False)  # no zero-filled gradient for an output the loss does not use
         cap = opts.get("capture")
         if cap is not None:
             cap.update(logits=logits, probs=probs, topk_idx=topk_idx, scores=scores, counts=counts, offsets=offsets,
@@ -212,7 +235,7 @@ class _ExpertLayerFn(torch.autograd.Function):
         return y, scores_out
 
     @staticmethod
-    def backward(ctx, dy, _ds_perm):
+    def backward(ctx, dy, ds_perm):
         (x, router_gate, w_gate_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, slot_of, scores_perm,
          gate_up, inter_s, sh_gate_up, sh_down, sh_out_gate, sh_gu, sh_inter_s, sh_sig) = ctx.saved_tensors
         opts = ctx.opts
@@ -220,9 +243,9 @@ class _ExpertLayerFn(torch.autograd.Function):
         T = x.shape[0]
         R = T * K
         cfg = opts["tile_cfg"]
-        if dy is None:  # the output took no part in the loss
+        if dy is None and ds_perm is None:  # neither output took part in the loss
             return (None,) * 9
-        dy = dy.contiguous()
+        dy = torch.zeros_like(x) if dy is None else dy.contiguous()
 
         # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMMs' loads
         ws = ctx.gemm_ws  # still holds the forward's tile map
@@ -238,11 +261,17 @@ class _ExpertLayerFn(torch.autograd.Function):
         d_w_gate_up = None
         if ctx.needs_input_grad[2]:
             d_w_gate_up = ops.grouped_gemm_wgrad(x, d_gate_up, offsets, E, tile_cfg=cfg, a_row_map=token_of)
+        if ds_perm is not None:
+            # gradient of the returned scores [R] (row order), taken back to the slots [T,K]
+            d_scores = d_scores + ds_perm.float()[row_of.long()]
 
         d_logits = ops.router_bwd(
             d_scores, probs, topk_idx, counts, x.dtype, opts["normalize"], opts["loss_coeff"] / T / opts["ep_size"]
         )
         d_router_gate = _router_weight_grad(d_logits, x) if ctx.needs_input_grad[1] else None
+        cap = opts.get("capture")
+        if cap is not None:
+            cap.update(d_scores=d_scores, d_logits=d_logits)
 
         d_sh_gate_up = d_sh_down = d_sh_out_gate = d_sh_gu = d_pre = None
         if ctx.shared:

@@ -339,11 +339,16 @@ def forward_backward(x, router_gate, expert_gate_up, expert_down, dy, cfg, **kw)
         t.detach().to(leaf_dtype).clone().requires_grad_(True) for t in (x, router_gate, expert_gate_up, expert_down)
     ]
     shared = kw.pop("shared", None)
+    d_scores_perm = kw.pop("d_scores_perm", None)  # upstream gradient of the returned scores (moe.py:323)
     if shared is not None:
         shared = tuple(t.detach().to(leaf_dtype).clone().requires_grad_(True) for t in shared)
     res = forward(*leaves, cfg, model_dtype=model_dtype, shared=shared, **kw)
     y = res["y"]
-    y.backward(dy.to(y.dtype).reshape(y.shape))
+    if d_scores_perm is None:
+        y.backward(dy.to(y.dtype).reshape(y.shape))
+    else:
+        sp = res["scores_perm"]
+        torch.autograd.backward([y, sp], [dy.to(y.dtype).reshape(y.shape), d_scores_perm.to(sp.dtype)])
     res["dx"], res["d_router_gate"], res["d_expert_gate_up"], res["d_expert_down"] = (t.grad for t in leaves)
     if shared is not None:
         res["d_shared_expert_gate_up"], res["d_shared_expert_down"], res["d_shared_expert_output_gate"] = (
@@ -355,6 +360,23 @@ def forward_backward(x, router_gate, expert_gate_up, expert_down, dy, cfg, **kw)
 def silu_grad(g: torch.Tensor) -> torch.Tensor:
     s = torch.sigmoid(g)
     return s * (1 + g * (1 - s))
+
+
+def router_backward(d_s_tk, probs, topk_idx, expert_freq, cfg, T):
+    """Gradient of the router from d(scores) [T,K] back to the logits: the derivative of the
+    normalisation and gather of moe.py:363-365, the load-balance hook moe.py:393-406 and the
+    softmax of moe.py:361.  Returns (d_probs, d_logits), both [T,E] in the dtype of probs."""
+    p_top = torch.gather(probs, -1, topk_idx)
+    if cfg.normalize_topk_scores:
+        S = p_top.sum(-1, keepdim=True)
+        sn = p_top / S
+        d_ptop = (d_s_tk - (d_s_tk * sn).sum(-1, keepdim=True)) / S
+    else:
+        d_ptop = d_s_tk
+    d_probs = torch.zeros_like(probs).scatter_add(-1, topk_idx, d_ptop)
+    d_probs = d_probs + expert_freq[None, :] * (cfg.loss_coeff / T) / cfg.ep_size
+    d_logits = probs * (d_probs - (probs * d_probs).sum(-1, keepdim=True))
+    return d_probs, d_logits
 
 
 def analytic_backward(res: Dict[str, torch.Tensor], x2d, router_gate, expert_gate_up, expert_down, dy2d, cfg):
@@ -403,18 +425,8 @@ def analytic_backward(res: Dict[str, torch.Tensor], x2d, router_gate, expert_gat
     d_s_flat = torch.zeros(T * K, dtype=dt)
     d_s_flat[perm] = d_s_perm
     d_s_tk = d_s_flat.view(K, T).t()
-    probs = res["probs"].detach().to(dt)
-    topk_idx = res["topk_idx"]
-    p_top = torch.gather(probs, -1, topk_idx)
-    if cfg.normalize_topk_scores:
-        S = p_top.sum(-1, keepdim=True)
-        sn = p_top / S
-        d_ptop = (d_s_tk - (d_s_tk * sn).sum(-1, keepdim=True)) / S
-    else:
-        d_ptop = d_s_tk
-    d_probs = torch.zeros_like(probs).scatter_add(-1, topk_idx, d_ptop)
-    d_probs = d_probs + res["expert_freq"].to(dt)[None, :] * (cfg.loss_coeff / T) / cfg.ep_size
-    d_logits = probs * (d_probs - (probs * d_probs).sum(-1, keepdim=True))
+    d_probs, d_logits = router_backward(d_s_tk, res["probs"].detach().to(dt), res["topk_idx"], res["expert_freq"].to(dt),
+                                        cfg, T)
     d_wr = d_logits.t() @ x2d
     dx = dx + d_logits @ router_gate
     return dict(

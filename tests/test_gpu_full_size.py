@@ -140,6 +140,64 @@ def test_full_size_layer(gpu_device, name):
                 assert err <= TOL, f"dW_gate_up[{e}][:, {c}]: {err:.3e}"
 
 
+@pytest.mark.parametrize("name", ["c3_qwen3_30b", "c5_stress"])
+def test_full_size_router_gradient(gpu_device, name):
+    """The router's gradient path at full size with the load-balance term switched on
+    (loss_coeff = 0.001): the score gradients of sampled tokens against their definition, the
+    router backward kernel against the oracle's formula on ALL tokens, and d_router_gate (the
+    16-way split of the token dimension on the weight-gradient kernel) against d_logits^T x in
+    float64."""
+    T, H, E, K, I, bias_hot, n_hot, n_dead, _ = FULL[name]
+    print("full-size router gradient", name, flush=True)
+    dev = gpu_device
+    x, wr, wgu, wd, dy = device_inputs(T, H, E, I, dev, 777, bias_hot, n_hot, n_dead)
+    layer = build_layer(torch.bfloat16, H, E, K, I, dev, loss_coeff=0.001)
+    with torch.no_grad():
+        layer.router_gate.copy_(wr)
+        layer.expert_gate_up.copy_(wgu)
+        layer.expert_down.copy_(wd)
+    layer.capture = {}
+    xg = x.clone().requires_grad_(True)
+    layer(xg).backward(dy)
+    torch.cuda.synchronize()
+    cap = layer.capture
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001)
+
+    # (a) score gradients of sampled tokens: d_s[t,k] = <dy[t], (up * act(gate)) @ W_down[e]>
+    act = O.activation("silu")
+    rng = np.random.default_rng(11)
+    topk = cap["topk_idx"].long()
+    S = np.sort(rng.choice(T, size=12, replace=False))
+    ref_ds = torch.zeros(len(S), K, dtype=torch.float64, device=dev)
+    for a, t in enumerate(S):
+        for k in range(K):
+            e = int(topk[t, k])
+            gu = bf16_round(x[t].double() @ wgu[e].double())
+            out = (gu[1::2] * act(gu[0::2])) @ wd[e].double()
+            ref_ds[a, k] = (dy[t].double() * out).sum()
+    err = O.rel_l2(cap["d_scores"][torch.from_numpy(S).to(dev)].cpu(), ref_ds.cpu())
+    print(f"  d_scores (sampled tokens): {err:.2e}", flush=True)
+    assert err <= TOL
+
+    # (b) router backward on all tokens from the captured score gradients
+    counts = cap["counts"].cpu().long()
+    freq = counts.double() / counts.sum().double()
+    _, ref_dl = O.router_backward(cap["d_scores"].cpu().double(), cap["probs"].cpu().double(), topk.cpu(), freq, ocfg, T)
+    err = O.rel_l2(cap["d_logits"].cpu(), ref_dl)
+    print(f"  d_logits (all tokens): {err:.2e}", flush=True)
+    assert err <= TOL
+    # (At this size the load-balance term, loss_coeff / T per entry and nearly uniform over the
+    # experts, lies below the float32 rounding of the softmax backward it is added into -- in the
+    # reference too; that it is applied is checked where it is visible, in
+    # test_layer_load_balance_term and test_router_bwd.)
+
+    # (c) d_router_gate = d_logits^T @ x, float64 on the device from the captured (bf16) d_logits
+    ref_wr = cap["d_logits"].double().t() @ x.double()
+    err = O.rel_l2(layer.router_gate.grad.cpu(), ref_wr.cpu())
+    print(f"  d_router_gate: {err:.2e}", flush=True)
+    assert err <= TOL
+
+
 def test_full_size_c4_grouped_gemms(ops, gpu_device):
     """C4: one EP rank's share of a DeepSeek-V3-like layer -- 65536 pre-assigned rows,
     32 local experts with Zipf(1.2) loads, H=7168, I=2048; forward and backward grouped GEMMs."""

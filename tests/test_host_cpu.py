@@ -1,0 +1,31 @@
+"""Host-side logic of the layer module that needs no GPU."""
+import torch
+
+from arctictraining_amd import moe
+
+
+def test_index_cache_is_bounded():
+    """Token counts change from step to step; the cache of split offsets must not grow with
+    the number of distinct sizes."""
+    cache = moe._INDEX_CACHE
+    for T in range(512, 1512):
+        offs = moe._token_offsets(T, 16, "cpu")
+        assert offs.dtype == torch.int32 and offs[0] == 0 and offs[-1] == T and offs.numel() == 17
+        assert bool((offs[1:] >= offs[:-1]).all())
+        ids = moe._token_ids(T, "cpu")
+        assert ids.numel() == T
+    assert len(cache) <= cache.max_entries
+    # a hit returns the cached tensor itself
+    a = moe._token_offsets(1511, 16, "cpu")
+    assert moe._token_offsets(1511, 16, "cpu") is a
+
+
+def test_activation_classification():
+    import torch.nn.functional as F
+
+    from arctictraining_amd import ops
+
+    assert moe.classify_activation(F.silu) == ops.ACT_SILU
+    assert moe.classify_activation(F.gelu) == ops.ACT_GELU
+    assert moe.classify_activation(F.relu) == ops.ACT_RELU
+    assert moe.classify_activation(lambda x: x * torch.sigmoid(1.702 * x)) == ops.ACT_GPT_OSS
