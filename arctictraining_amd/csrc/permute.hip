@@ -8,6 +8,8 @@
 // order inside an expert is ascending f by construction, with no global atomics.
 #include "amoe_common.h"
 
+#include <atomic>
+
 namespace {
 
 constexpr int kChunk = 512;         // flat slots per wavefront
@@ -141,23 +143,28 @@ AMOE_EXPORT size_t amoe_permute_workspace_bytes(int R, int E)
     return (size_t)permute_chunks(R) * (size_t)E * sizeof(int32_t);
 }
 
-AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
-                                  int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of,
-                                  float* scores_perm, void* workspace, size_t workspace_bytes, void* stream)
+// argument checks shared by the two entry points (all before the first HIP call)
+static int check_plan_args(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                           int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of, float* scores_perm)
 {
-    AMOE_REQUIRE(assign && counts && offsets && token_of && slot_of && row_of && workspace, AMOE_ERR_BAD_ARG,
+    AMOE_REQUIRE(assign && counts && offsets && token_of && slot_of && row_of, AMOE_ERR_BAD_ARG,
                  "permute_plan: null pointer");
     AMOE_REQUIRE(!scores_perm || scores, AMOE_ERR_BAD_ARG, "permute_plan: scores_perm needs scores");
     AMOE_REQUIRE(T > 0 && K > 0 && E > 0, AMOE_ERR_BAD_ARG, "permute_plan: T, K, E must be positive");
     AMOE_REQUIRE(E <= AMOE_MAX_EXPERTS, AMOE_ERR_UNSUPPORTED, "permute_plan: E=%d exceeds %d", E, AMOE_MAX_EXPERTS);
     AMOE_REQUIRE((long long)T * K < (1ll << 31), AMOE_ERR_UNSUPPORTED, "permute_plan: T*K does not fit int32");
+    return AMOE_OK;
+}
+
+// the three launches; cc = per-chunk expert counts, permute_chunks(R) * E int32 (every entry is
+// written by the histogram kernel before it is read: nothing has to be cleared)
+static int launch_plan(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                       int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of, float* scores_perm,
+                       int32_t* cc, hipStream_t s)
+{
     const int R = T * K;
-    AMOE_REQUIRE(workspace_bytes >= amoe_permute_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
-                 "permute_plan: workspace %zu < %zu bytes", workspace_bytes, amoe_permute_workspace_bytes(R, E));
     const int n_chunks = permute_chunks(R);
     const int n_blocks = (n_chunks + kWavesPerBlock - 1) / kWavesPerBlock;
-    hipStream_t s = (hipStream_t)stream;
-    int32_t* cc = (int32_t*)workspace;
     hipLaunchKernelGGL(permute_hist_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E, R,
                        n_chunks, cc);
     int EP = 1;
@@ -166,4 +173,69 @@ AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, const float* scores, in
     hipLaunchKernelGGL(permute_scatter_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E,
                        R, n_chunks, cc, offsets, scores, token_of, slot_of, row_of, scores_perm);
     return amoe_check_launch("permute_plan");
+}
+
+AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                                  int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of,
+                                  float* scores_perm, void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = check_plan_args(assign, scores, T, K, E, counts, offsets, token_of, slot_of, row_of, scores_perm);
+    if (rc) return rc;
+    AMOE_REQUIRE(workspace, AMOE_ERR_BAD_ARG, "permute_plan: null workspace");
+    AMOE_REQUIRE(workspace_bytes >= amoe_permute_workspace_bytes(T * K, E), AMOE_ERR_WORKSPACE,
+                 "permute_plan: workspace %zu < %zu bytes", workspace_bytes, amoe_permute_workspace_bytes(T * K, E));
+    return launch_plan(assign, scores, T, K, E, counts, offsets, token_of, slot_of, row_of, scores_perm,
+                       (int32_t*)workspace, (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------ the variant that allocates nothing
+// The per-chunk counts live in a fixed array in device memory that belongs to the library (each
+// GPU the library runs on holds its own copy until the process ends).  Host code never uses the
+// array's name as an address: the device address is looked up once per device and kept.
+static __device__ __align__(256) int32_t scratch[AMOE_PERMUTE_STATIC_MAX_COUNTS];
+
+static constexpr int kMaxDevices = 64;
+static std::atomic<int32_t*> g_scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device (resolved on the first call per device)
+static int static_scratch(int32_t** out)
+{
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        amoe_set_error("permute_plan_static: no usable current device (%s)", hipGetErrorString(err));
+        return AMOE_ERR_LAUNCH;
+    }
+    int32_t* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        void* sym = nullptr;
+        err = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !sym) {
+            amoe_set_error("permute_plan_static: cannot resolve the scratch array on device %d: %s", dev,
+                           hipGetErrorString(err));
+            return AMOE_ERR_LAUNCH;
+        }
+        ptr = (int32_t*)sym;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // racing threads store the same address
+    }
+    *out = ptr;
+    return AMOE_OK;
+}
+
+AMOE_EXPORT int amoe_permute_plan_static(const int32_t* assign, const float* scores, int T, int K, int E,
+                                         int32_t* counts, int32_t* offsets, int32_t* token_of, int32_t* slot_of,
+                                         int32_t* row_of, float* scores_perm, void* stream)
+{
+    int rc = check_plan_args(assign, scores, T, K, E, counts, offsets, token_of, slot_of, row_of, scores_perm);
+    if (rc) return rc;
+    const long long need = (long long)permute_chunks(T * K) * E;
+    AMOE_REQUIRE(need <= (long long)AMOE_PERMUTE_STATIC_MAX_COUNTS, AMOE_ERR_UNSUPPORTED,
+                 "permute_plan_static: ceil(T*K/%d)*E = %lld exceeds the built-in scratch of %d counters; "
+                 "use amoe_permute_plan with a caller workspace",
+                 kChunk, need, AMOE_PERMUTE_STATIC_MAX_COUNTS);
+    int32_t* cc = nullptr;
+    rc = static_scratch(&cc);
+    if (rc) return rc;
+    return launch_plan(assign, scores, T, K, E, counts, offsets, token_of, slot_of, row_of, scores_perm, cc,
+                       (hipStream_t)stream);
 }

@@ -102,6 +102,29 @@ def permute_plan(assign: torch.Tensor, num_experts: int, scores: Optional[torch.
     return counts, offsets, token_of, slot_of, row_of, scores_perm
 
 
+def permute_plan_static(assign: torch.Tensor, num_experts: int, scores: Optional[torch.Tensor] = None, out=None):
+    """permute_plan through the entry point that allocates nothing: its counters live in a fixed
+    array inside the library (ceil(T*K/512)*E <= 2^20).  `out` = (counts, offsets, token_of, slot_of,
+    row_of, scores_perm) preallocated by the caller makes the call itself allocation-free."""
+    lib = _lib.load()
+    _chk(assign, "assign", torch.int32)
+    T, K = assign.shape
+    R, E, dev = T * K, num_experts, assign.device
+    if out is None:
+        i32 = dict(dtype=torch.int32, device=dev)
+        out = (torch.empty(E, **i32), torch.empty(E + 1, **i32), torch.empty(R, **i32), torch.empty(R, **i32),
+               torch.empty((T, K), **i32), torch.empty(R, dtype=torch.float32, device=dev) if scores is not None else None)
+    counts, offsets, token_of, slot_of, row_of, scores_perm = out
+    if scores is not None:
+        _chk(scores, "scores", torch.float32)
+    rc = lib.amoe_permute_plan_static(
+        assign.data_ptr(), _ptr(scores), T, K, E, counts.data_ptr(), offsets.data_ptr(), token_of.data_ptr(),
+        slot_of.data_ptr(), row_of.data_ptr(), _ptr(scores_perm) if scores is not None else None, _stream()
+    )
+    _lib.check(rc, "amoe_permute_plan_static")
+    return counts, offsets, token_of, slot_of, row_of, (scores_perm if scores is not None else None)
+
+
 def gather_rows_fwd(x: torch.Tensor, token_of: torch.Tensor) -> torch.Tensor:
     lib = _lib.load()
     _chk(x, "x")

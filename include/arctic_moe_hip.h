@@ -90,6 +90,24 @@ int amoe_permute_plan(const int32_t* assign, const float* scores, int T, int K, 
                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * amoe_permute_plan for callers that cannot allocate device memory (code recorded into a HIP
+ * graph, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results as amoe_permute_plan without the workspace: the
+ * per-chunk counters live in a fixed array of AMOE_PERMUTE_STATIC_MAX_COUNTS int32 (4 MiB) in
+ * device memory that the library owns on every GPU it runs on until the process ends.  The call
+ * allocates and frees nothing.  Limit: ceil(T*K/512) * E <= AMOE_PERMUTE_STATIC_MAX_COUNTS
+ * (e.g. T*K = 1M routed rows at E = 512, or 4M at E = 128); beyond it AMOE_ERR_UNSUPPORTED.
+ * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two
+ * threads) race; calls ordered on one stream are safe.  The first call on a device looks up the
+ * array's device address (a host-side query, not a stream operation), so make it once before
+ * recording a graph.
+ */
+#define AMOE_PERMUTE_STATIC_MAX_COUNTS (1 << 20)
+int amoe_permute_plan_static(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                             int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of,
+                             float* scores_perm, void* stream);
+
+/*
  * Row gather  xp[r,:] = x[token_of[r],:]  (moe.py:356; forward half of moe_scatter,
  * moe_scatter_cuda.cu:141-154).  x [T,H], xp [R,H].
  */

@@ -74,6 +74,15 @@ def test_permute_argument_errors(lib):
     assert lib.amoe_permute_plan(P, None, 4, 2, 600, P, P, P, P, P, None, P, 1 << 20, None) == -2
 
 
+def test_permute_static_argument_errors(lib):
+    assert lib.amoe_permute_plan_static(None, None, 4, 2, 8, P, P, P, P, P, None, None) == -1
+    assert lib.amoe_permute_plan_static(P, None, 4, 2, 8, P, P, P, P, P, P, None) == -1  # scores_perm without scores
+    assert lib.amoe_permute_plan_static(P, None, 4, 2, 600, P, P, P, P, P, None, None) == -2  # E too large
+    # ceil(T*K/512) * E beyond the built-in scratch of 2^20 counters: rejected before any HIP call
+    assert lib.amoe_permute_plan_static(P, None, 1 << 20, 2, 512, P, P, P, P, P, None, None) == -2
+    assert b"scratch" in lib.amoe_last_error()
+
+
 def test_row_kernel_argument_errors(lib):
     assert lib.amoe_gather_rows_fwd(P, P, P, 1, 8, 12, None) == -2  # bf16 row not a multiple of 8
     assert lib.amoe_gather_rows_fwd(P, P, P, 0, 8, 6, None) == -2  # f32 row not a multiple of 4
