@@ -269,6 +269,8 @@ GEMM_CASES = [
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 2),
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 3),
     (torch.bfloat16, 1000, 8, 128, 192, "ragged", 5),
+    (torch.bfloat16, 1500, 3, 448, 704, "ragged", 0),
+    (torch.bfloat16, 2100, 9, 832, 256, "holes", 0),
     (torch.bfloat16, 3000, 5, 320, 576, "ragged", 0),
     (torch.bfloat16, 3000, 5, 320, 576, "holes", 5),
     (torch.bfloat16, 777, 6, 256, 320, "holes", 0),
