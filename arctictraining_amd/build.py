@@ -55,8 +55,18 @@ def _compile(src: str) -> str:
     return obj
 
 
+def _check_gemm_assembly() -> None:
+    """Compile gemm_bf16.hip to assembly and run the static check of its inline-assembly LDS
+    reads (asm_check.py); raises, and so fails the build, on a violation."""
+    from . import asm_check
+
+    flags = [f for f in HIPCC_FLAGS if f not in ("-fPIC", "-fvisibility=hidden")]
+    asm = asm_check.compile_to_assembly(os.path.join(SRC_DIR, "gemm_bf16.hip"), os.path.join(OBJ_DIR, "gemm_bf16.s"), flags)
+    asm_check.check_assembly(asm, min_kernels=20)
+
+
 def build(force: bool = True, jobs: int = 6) -> str:
-    """Compile every HIP source and link the shared library; returns its path."""
+    """Compile every HIP source, check the GEMM assembly, and link the shared library; returns its path."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     if not force and os.path.exists(LIB_PATH):
@@ -68,8 +78,10 @@ def build(force: bool = True, jobs: int = 6) -> str:
         )
         if os.path.getmtime(LIB_PATH) >= newest:
             return LIB_PATH
-    with ThreadPoolExecutor(max_workers=jobs) as ex:
+    with ThreadPoolExecutor(max_workers=jobs + 1) as ex:
+        check = ex.submit(_check_gemm_assembly)
         objs = list(ex.map(_compile, SOURCES))
+        check.result()  # a violation raises here: no library is linked from a source that fails the check
     cmd = [hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

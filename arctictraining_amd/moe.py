@@ -9,6 +9,7 @@ The whole routed-expert computation is one torch.autograd.Function whose forward
 backward call the kernels stage by stage with no host synchronisation.
 """
 import contextlib
+import os
 import time
 from collections import OrderedDict, defaultdict
 from dataclasses import dataclass
@@ -173,7 +174,16 @@ class _ExpertLayerFn(torch.autograd.Function):
         timers.start("router")
         logits = torch.matmul(x, router_gate.t())  # plain library GEMM, moe.py:233
         probs, topk_idx, scores = ops.router_topk_fwd(logits, K, opts["normalize"])
-        assign = topk_idx if replay is None else replay.to(torch.int32).contiguous()
+        assign = topk_idx
+        if replay is not None:
+            assign = replay.to(torch.int32).contiguous()
+            if os.environ.get("AMOE_CHECK_REPLAY") == "1":
+                # The reference's one_hot(..., num_classes=E) raises on an expert id outside [0, E)
+                # (moe.py:374); the permutation kernels clamp such ids for memory safety instead.  This
+                # opt-in check restores the error at the price of a host synchronisation.
+                bad = ((assign < 0) | (assign >= E)).any()
+                if bool(bad):
+                    raise RuntimeError(f"routing_replay_assignments holds expert ids outside [0, {E})")
         counts, offsets, token_of, slot_of, row_of, scores_perm = ops.permute_plan(assign, E, scores)
         timers.stop("router")
 

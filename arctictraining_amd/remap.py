@@ -10,11 +10,15 @@ The weight re-layout itself -- transposing each expert's nn.Linear weights and i
 gate / up on the last dimension -- runs in the HIP kernels of csrc/remap.hip through the C ABI
 (`amoe_remap_pack`, `amoe_remap_unpack`); there is no torch or CPU fallback for it.
 
-Two storage formats of the original experts are understood:
+Three storage formats of the original experts are understood:
   * a ModuleList of per-expert MLPs with `gate_proj`, `up_proj`, `down_proj` nn.Linear modules
     (what the reference reads, utils.py:232-254);
   * fused tensors `experts.gate_up_proj [E, 2I, H]` (gate rows, then up rows) and
-    `experts.down_proj [E, H, I]` (the Qwen3-MoE experts of transformers >= 5).
+    `experts.down_proj [E, H, I]` (the Qwen3-MoE experts of transformers >= 5);
+  * the gpt-oss experts (the reference's non-list branch, utils.py:291-299): `gate_up_proj` holds
+    gate and up INTERLEAVED, either as [E, 2I, H] (the reference transposes it) or already as
+    [E, H, 2I]; `down_proj [E, H, I]`.  Which fused format a model uses is decided by its
+    architecture (`fused_gate_up_interleaved` of the derived config), never guessed from shapes.
 """
 import copy
 import re
@@ -62,6 +66,7 @@ def arctic_moe_config_from_hf(config, dtype, ep_size=1, enable_routing_replay=Fa
         )
     ns.use_shared_expert = hasattr(config, "shared_expert_intermediate_size")
     ns.return_router_scores = arch in ("GptOssForCausalLM",)
+    ns.fused_gate_up_interleaved = "GptOss" in arch  # layout of a fused experts.gate_up_proj tensor
     ns.use_triton = False
     ns.is_gated = True
     ns.use_custom_moe_kernel = False
@@ -89,10 +94,26 @@ def fill_arctic_moe_from_orig_mlp(arctic_moe: ArcticMoE, orig_mlp, device) -> No
         up = _stacked_linear_weights(experts, "up_proj", device)
         down = _stacked_linear_weights(experts, "down_proj", device)  # [E, H, I]
     else:
-        fused = experts.gate_up_proj.detach().to(device)  # [E, 2I, H]: gate rows, then up rows
+        fused = experts.gate_up_proj.detach().to(device)
+        down = experts.down_proj.detach().to(device).contiguous()
+        H, I2 = arctic_moe.model_dim, 2 * arctic_moe.intermediate_dim
+        if getattr(arctic_moe._config, "fused_gate_up_interleaved", False):
+            # gpt-oss: gate / up already interleaved; at most a batched transpose is needed
+            if tuple(fused.shape[-2:]) == (I2, H) and H != I2:
+                arctic_moe.expert_gate_up.copy_(ops.remap_pack(fused.contiguous()))
+            elif tuple(fused.shape[-2:]) == (H, I2):
+                arctic_moe.expert_gate_up.copy_(fused)
+            else:
+                raise ValueError(f"gate_up_proj of shape {tuple(fused.shape)} is neither [E, {I2}, {H}] nor [E, {H}, {I2}]")
+            arctic_moe.expert_down.copy_(ops.remap_pack(down))
+            return
+        if tuple(fused.shape[-2:]) != (I2, H):
+            raise ValueError(
+                f"fused gate_up_proj of shape {tuple(fused.shape)}: expected [E, {I2}, {H}] (gate rows, then up rows); "
+                "a tensor that interleaves gate and up (gpt-oss) needs fused_gate_up_interleaved=True in the config"
+            )
         inter = fused.shape[1] // 2
         gate, up = fused[:, :inter, :], fused[:, inter:, :]
-        down = experts.down_proj.detach().to(device).contiguous()
     arctic_moe.expert_gate_up.copy_(ops.remap_pack(gate, up))
     arctic_moe.expert_down.copy_(ops.remap_pack(down))
     if arctic_moe._config.use_shared_expert:
@@ -117,6 +138,14 @@ def fill_orig_mlp_from_arctic_moe(orig_mlp, arctic_moe: ArcticMoE) -> None:
             ex.gate_proj.weight.copy_(gate[i])
             ex.up_proj.weight.copy_(up[i])
             ex.down_proj.weight.copy_(down[i])
+    elif getattr(arctic_moe._config, "fused_gate_up_interleaved", False):
+        fused = experts.gate_up_proj
+        H, I2 = arctic_moe.model_dim, 2 * arctic_moe.intermediate_dim
+        if tuple(fused.shape[-2:]) == (I2, H) and H != I2:
+            fused.copy_(ops.remap_unpack(gate_up, two=False))
+        else:
+            fused.copy_(gate_up)
+        experts.down_proj.copy_(down)
     else:
         fused = experts.gate_up_proj
         inter = fused.shape[1] // 2

@@ -154,6 +154,19 @@ def test_layer_routing_replay_and_returned_scores(gpu_device):
     assert O.rel_l2(scores.cpu(), ref["scores_perm"]) <= 1e-2
     with pytest.raises(AssertionError):
         layer(x.to(gpu_device))
+    # an expert id outside [0, E): clamped by default (no host sync on the hot path); the opt-in
+    # check restores the error the reference's one_hot raises (moe.py:374)
+    bad = replay.clone()
+    bad[5, 0] = E + 3
+    import os
+    layer(x.to(gpu_device), bad.to(gpu_device))
+    torch.cuda.synchronize()
+    os.environ["AMOE_CHECK_REPLAY"] = "1"
+    try:
+        with pytest.raises(RuntimeError, match="outside"):
+            layer(x.to(gpu_device), bad.to(gpu_device))
+    finally:
+        del os.environ["AMOE_CHECK_REPLAY"]
 
 
 @pytest.mark.parametrize(

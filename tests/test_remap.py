@@ -263,3 +263,73 @@ def test_install_and_restore_hooks_shared_expert(gpu_device):
     assert got.keys() == saved.keys()
     for k in saved:
         assert torch.equal(got[k], saved[k]), k
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("transposed", [True, False])
+def test_install_and_restore_hooks_gpt_oss_layout(gpu_device, transposed):
+    """The reference's non-list branch (utils.py:291-299): fused experts whose gate_up_proj
+    INTERLEAVES gate and up, stored [E, 2I, H] (transposed on install) or already [E, H, 2I].
+    The installed layer must hold exactly gate in the even and up in the odd columns."""
+    from types import SimpleNamespace
+
+    from arctictraining_amd import ArcticMoE
+    from arctictraining_amd.remap import remap_arctic_moe_to_orig_moe_mlp_params, remap_orig_moe_mlp_params_to_arctic_moe
+
+    E, K, H, I = 4, 2, 64, 48
+    g = torch.Generator().manual_seed(8)
+    gate_w, up_w = torch.randn(E, H, I, generator=g), torch.randn(E, H, I, generator=g)   # [in, out]
+    interleaved = torch.stack((gate_w, up_w), dim=-1).reshape(E, H, 2 * I)                # ArcticMoE layout
+    down_w = torch.randn(E, H, I, generator=g)                                            # nn.Linear layout [out, in]
+    experts = torch.nn.Module()
+    experts.gate_up_proj = torch.nn.Parameter((interleaved.transpose(1, 2) if transposed else interleaved).contiguous())
+    experts.down_proj = torch.nn.Parameter(down_w.clone())
+    mlp = torch.nn.Module()
+    mlp.gate = torch.nn.Linear(H, E, bias=False)
+    mlp.experts = experts
+    mlp = mlp.to(gpu_device)
+    saved = {k: v.detach().clone() for k, v in mlp.state_dict().items()}
+    layer = torch.nn.Module()
+    layer.mlp = mlp
+    model = torch.nn.Module()
+    model.model = torch.nn.Module()
+    model.model.layers = torch.nn.ModuleList([layer])
+    model.config = SimpleNamespace(hidden_size=H, num_experts_per_tok=K, router_aux_loss_coef=0.0, hidden_act="silu",
+                                   intermediate_size=I, num_local_experts=E, architectures=["GptOssForCausalLM"])
+    model.dtype = torch.float32
+    remap_orig_moe_mlp_params_to_arctic_moe(model, device=gpu_device)
+    amoe = model.model.layers[0].mlp
+    assert isinstance(amoe, ArcticMoE) and amoe._config.return_router_scores
+    assert torch.equal(amoe.expert_gate_up.detach().cpu(), interleaved)
+    assert torch.equal(amoe.expert_down.detach().cpu(), down_w.transpose(1, 2))
+    remap_arctic_moe_to_orig_moe_mlp_params(model)
+    got = model.model.layers[0].mlp.state_dict()
+    for k in saved:
+        assert torch.equal(got[k], saved[k]), k
+
+
+@pytest.mark.gpu
+def test_fused_layout_mismatch_is_an_error(gpu_device):
+    """A fused gate_up_proj that does not have the [E, 2I, H] shape of the architecture's format
+    raises instead of being misread."""
+    from types import SimpleNamespace
+
+    from arctictraining_amd.remap import remap_orig_moe_mlp_params_to_arctic_moe
+
+    E, K, H, I = 4, 2, 64, 48
+    experts = torch.nn.Module()
+    experts.gate_up_proj = torch.nn.Parameter(torch.zeros(E, H, 2 * I))   # gpt-oss layout under a Qwen architecture
+    experts.down_proj = torch.nn.Parameter(torch.zeros(E, H, I))
+    mlp = torch.nn.Module()
+    mlp.gate = torch.nn.Linear(H, E, bias=False)
+    mlp.experts = experts
+    layer = torch.nn.Module()
+    layer.mlp = mlp.to(gpu_device)
+    model = torch.nn.Module()
+    model.model = torch.nn.Module()
+    model.model.layers = torch.nn.ModuleList([layer])
+    model.config = SimpleNamespace(hidden_size=H, num_experts_per_tok=K, router_aux_loss_coef=0.0, hidden_act="silu",
+                                   moe_intermediate_size=I, num_experts=E, architectures=["Qwen3MoeForCausalLM"])
+    model.dtype = torch.float32
+    with pytest.raises(ValueError, match="interleaves"):
+        remap_orig_moe_mlp_params_to_arctic_moe(model, device=gpu_device)
