@@ -63,6 +63,13 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
          _c_void_p],
     ),
+    "amoe_gated_bwd_score_parts": (_c_int, [_c_int, _c_int]),
+    "amoe_grouped_gemm_nt_gated_bwd": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_void_p, _c_size_t, _c_int, _c_void_p],
+    ),
+    "amoe_score_grad_gather": (_c_int, [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p]),
     "amoe_remap_pack": (
         _c_int,
         [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, ctypes.c_longlong, _c_void_p],

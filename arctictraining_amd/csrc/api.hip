@@ -27,6 +27,10 @@ int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const i
                  int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s);
 int amoe_bf16_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
                     const int32_t* offsets, void* C, int R, int E, int Kd, int N, int tile_cfg, hipStream_t s);
+int amoe_bf16_nt_gated_bwd(const void* dy, const int32_t* a_row_map, const void* w_down, const int32_t* offsets,
+                           const void* gate_up, const float* row_scale, void* d_gate_up, float* partials, int R, int E,
+                           int I, int H, int act, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s);
+int amoe_bf16_gated_bwd_parts(int I, int tile_cfg);
 int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                   int Kred, int N, int ldb, long long strideB, bool b_kc, void* workspace, size_t workspace_bytes,
                   hipStream_t s);
@@ -150,4 +154,32 @@ AMOE_EXPORT int amoe_grouped_gemm_wgrad(const void* A, const int32_t* a_row_map,
     hipStream_t s = (hipStream_t)stream;
     if (dtype == AMOE_BF16) return amoe_bf16_wgrad(A, a_row_map, B, b_row_map, offsets, C, R, E, Kd, N, tile_cfg, s);
     return amoe_f32_wgrad(A, a_row_map, B, b_row_map, offsets, C, R, E, Kd, N, s);
+}
+
+AMOE_EXPORT int amoe_gated_bwd_score_parts(int I, int tile_cfg)
+{
+    if (I <= 0 || tile_cfg < 0) return 0;
+    return amoe_bf16_gated_bwd_parts(I, tile_cfg);
+}
+
+AMOE_EXPORT int amoe_grouped_gemm_nt_gated_bwd(const void* dy, const int32_t* a_row_map, const void* w_down,
+                                               const int32_t* offsets, const void* gate_up, const float* row_scale,
+                                               void* d_gate_up, float* score_partials, int dtype, int R, int E, int I,
+                                               int H, int act, void* workspace, size_t workspace_bytes, int tile_cfg,
+                                               void* stream)
+{
+    const char* what = "grouped_gemm_nt_gated_bwd";
+    AMOE_REQUIRE(dy && w_down && offsets && gate_up && d_gate_up && workspace, AMOE_ERR_BAD_ARG, "%s: null pointer", what);
+    int rc = check_gemm_common(what, dtype, R, E, I, H, tile_cfg);
+    if (rc) return rc;
+    AMOE_REQUIRE(dtype == AMOE_BF16, AMOE_ERR_UNSUPPORTED,
+                 "%s: bf16 only (float32 callers run amoe_grouped_gemm_nt and amoe_gated_act_bwd)", what);
+    AMOE_REQUIRE(act >= AMOE_ACT_SILU && act <= AMOE_ACT_GPT_OSS, AMOE_ERR_BAD_ARG, "%s: bad activation %d", what, act);
+    AMOE_REQUIRE((long long)R * 2 * I < (1ll << 32), AMOE_ERR_UNSUPPORTED, "%s: an operand exceeds 2^32 elements", what);
+    rc = check_gemm_dims(what, dtype, H, I);  // the reduction runs over H
+    if (rc) return rc;
+    AMOE_REQUIRE(workspace_bytes >= amoe_grouped_gemm_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
+                 "%s: workspace %zu < %zu bytes", what, workspace_bytes, amoe_grouped_gemm_workspace_bytes(R, E));
+    return amoe_bf16_nt_gated_bwd(dy, a_row_map, w_down, offsets, gate_up, row_scale, d_gate_up, score_partials, R, E, I, H,
+                                  act, workspace, workspace_bytes, tile_cfg, (hipStream_t)stream);
 }

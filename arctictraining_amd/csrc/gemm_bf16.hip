@@ -50,7 +50,10 @@ struct GemmArgs {
     bf16_t* C2;
     const int32_t* a_row_map;
     const int32_t* b_row_map;  // weight gradient only
-    const float* row_scale;  // gated epilogue: inter[r,:] is multiplied by row_scale[r] (null = 1)
+    const float* row_scale;  // gated epilogues: the per-row factor of the gated activation (null = 1)
+    const bf16_t* G;         // gated-backward epilogue: gate_up [R, 2N] of the forward pass
+    float* partials;         // gated-backward epilogue: [n_ntiles][part_stride] row sums, or null
+    int ldg, part_stride;
     const int32_t* offsets;
     const int4* tile_map;
     const int32_t* n_mtiles;
@@ -68,7 +71,7 @@ struct GemmArgs {
     int max_mtiles;  // rows mode: entries of tile_map (those past the last tile hold expert -1)
 };
 
-enum { EPI_STORE = 0, EPI_GATED = 1 };
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_GATED_BWD = 2 };
 
 // tile map: one int4 {expert, first row, end row, 0} per M tile
 __global__ void __launch_bounds__(512)
@@ -162,6 +165,20 @@ __device__ __forceinline__ float act_fwd_fast(float g)
     if (ACT == AMOE_ACT_GPT_OSS) return g * __builtin_amdgcn_rcpf(1.0f + __expf(-1.702f * g));
     return act_fwd<ACT>(g);
 }
+// act(g) and act'(g) for the backward epilogue, sharing one sigmoid (hardware reciprocal, see above)
+template <int ACT>
+__device__ __forceinline__ void act_both_fast(float g, float& f, float& df)
+{
+    if (ACT == AMOE_ACT_SILU || ACT == AMOE_ACT_GPT_OSS) {
+        const float a = ACT == AMOE_ACT_SILU ? 1.0f : 1.702f;
+        const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-a * g));
+        f = g * sg;
+        df = sg * (1.0f + a * g * (1.0f - sg));
+    } else {
+        f = act_fwd<ACT>(g);
+        df = act_bwd<ACT>(g);
+    }
+}
 using T_ = std::true_type;
 using F_ = std::false_type;
 
@@ -243,7 +260,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     // vector loads between the stores, and a load result can only be awaited together with every
     // store issued before it.
     float rs_in = 1.0f;
-    if (EPI == EPI_GATED && tid < BM && p.row_scale) rs_in = p.row_scale[min(m0 + tid, mend - 1)];
+    if (EPI != EPI_STORE && tid < BM && p.row_scale) rs_in = p.row_scale[min(m0 + tid, mend - 1)];
 #pragma unroll
     for (int i = 0; i < PER_A; ++i) {
         const int c = tid + NT * i;
@@ -600,7 +617,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     bf16_t* Cb = WGRAD ? p.C + (long long)e * p.strideC : p.C;
     const int odd1 = lj & 1, odd2 = (lj >> 1) & 1;
     float* s_rs = reinterpret_cast<float*>(smem);   // the stages are free once every wave is past the loop
-    if (EPI == EPI_GATED) {
+    if (EPI != EPI_STORE) {
         __syncthreads();
         if (tid < BM) s_rs[tid] = rs_in;
         __syncthreads();
@@ -662,6 +679,103 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             }
         }
     };
+    if (EPI == EPI_GATED_BWD) {
+        // The accumulators are d_inter[r, c] (c = intermediate column); nothing of it is stored.
+        // With (gate, up) = gate_up[r, 2c], gate_up[r, 2c+1] re-read from the forward pass and
+        // s = row_scale[r]:  d_gate_up[r, 2c] = s * d * up * act'(gate),  d_gate_up[r, 2c+1] =
+        // s * d * act(gate)  (one packed pair per element, no lane exchange needed), and the row
+        // sums  sum_c d * up * act(gate)  -- the gradient of s -- are reduced over the tile's columns
+        // in a fixed order and written to partials[N tile][row].
+        float* s_part = s_rs + BM;   // [2 * WGN][BM] partial row sums of the half-wave column groups
+        // gate_up and d_gate_up have the same [R, 2N] shape: one wave-uniform origin each (scalar
+        // arithmetic per element row) plus one per-lane byte offset shared by both
+        const long long gorg = (long long)(m0 + wm * WTM) * p.ldg + 2 * (n0 + wn * WTN);
+        const char* gbase = reinterpret_cast<const char*>(p.G + gorg);
+        char* dbase = reinterpret_cast<char*>(p.C + gorg);
+        const uint32_t goff = (uint32_t)(4 * lg * p.ldg + 2 * lj) * 2u;
+        auto run = [&](auto FULL) {
+            constexpr bool full = decltype(FULL)::value;
+            // a block = 8 of the 16 values a lane holds of one 32x32 tile (half hh: registers 8hh..8hh+7)
+            auto load_block = [&](int i, int j, int hh, uint32_t (&g)[8]) {
+                const bool col_ok = full || (n0 + wn * WTN + j * 32 + lj < p.N);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int v = 8 * hh + u;
+                    const int rr = i * 32 + 8 * (v >> 2) + (v & 3);   // row relative to the wave's origin (+ 4*lg in goff)
+                    const bool ok = full || (col_ok && m0 + wm * WTM + rr + 4 * lg < mend);
+                    const char* rowp = gbase + ((long long)rr * p.ldg + 2 * j * 32) * 2;
+                    g[u] = ok ? *reinterpret_cast<const uint32_t*>(rowp + goff) : 0u;
+                }
+            };
+            uint32_t gcur[8], gnxt[8];
+            load_block(0, 0, 0, gcur);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                float dot[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) dot[v] = 0.f;
+#pragma unroll
+                for (int jh = 0; jh < 2 * TN; ++jh) {
+                    const int j = jh >> 1, hh = jh & 1;
+                    // the next block's pairs are requested before this block is worked on
+                    constexpr int NB = TM * TN * 2;
+                    const int b_next = i * 2 * TN + jh + 1;
+                    if (b_next < NB) load_block(b_next / (2 * TN), (b_next % (2 * TN)) >> 1, b_next & 1, gnxt);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const bool col_ok = full || (n0 + wn * WTN + j * 32 + lj < p.N);
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        // (fenced every four elements: left alone, the scheduler interleaves all the
+                        // activation chains and their temporaries no longer fit beside the accumulators)
+                        if (u == 4) __builtin_amdgcn_sched_barrier(0);
+                        const int v = 8 * hh + u;
+                        const int rr = i * 32 + 8 * (v >> 2) + (v & 3);
+                        const float d = acc[i][j][v];
+                        const float gate = bf16_lo(gcur[u]), up = bf16_hi(gcur[u]);
+                        float f, df;
+                        act_both_fast<ACT>(gate, f, df);
+                        const float sd = s_rs[wm * WTM + rr + 4 * lg] * d;
+                        dot[v] += d * up * f;
+                        const bool ok = full || (col_ok && m0 + wm * WTM + rr + 4 * lg < mend);
+                        if (ok) {
+                            char* rowp = dbase + ((long long)rr * p.ldg + 2 * j * 32) * 2;
+                            *reinterpret_cast<uint32_t*>(rowp + goff) = pack_bf16x2(sd * up * df, sd * f);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (b_next < NB) {
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) gcur[u] = gnxt[u];
+                    }
+                }
+                if (p.partials) {
+                    // sum over the 16 lanes of a row group (its 16 columns), then one slot per
+                    // (wave column, half-wave group) and tile row
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        float x = dot[v];
+                        x += dpp_f32<AMOE_DPP_QUAD_XOR1>(x);
+                        x += dpp_f32<AMOE_DPP_QUAD_XOR2>(x);
+                        x += dpp_f32<AMOE_DPP_HALF_MIRROR>(x);
+                        x += dpp_f32<AMOE_DPP_MIRROR>(x);
+                        if ((lane & 15) == 0)
+                            s_part[(wn * 2 + ((lane >> 4) & 1)) * BM + wm * WTM + i * 32 + 8 * (v >> 2) + 4 * lg + (v & 3)] = x;
+                    }
+                }
+            }
+        };
+        if (m0 + BM <= mend && n0 + BN <= p.N) run(T_{}); else run(F_{});
+        if (p.partials) {
+            __syncthreads();
+            if (tid < BM && m0 + tid < mend) {
+                float tot = 0.f;
+#pragma unroll
+                for (int q = 0; q < 2 * WGN; ++q) tot += s_part[q * BM + tid];
+                p.partials[(long long)nt * p.part_stride + m0 + tid] = tot;
+            }
+        }
+        return;
+    }
     if (m0 + BM <= mend && n0 + BN <= p.N) epilogue(T_{}); else epilogue(F_{});
 }
 
@@ -709,8 +823,22 @@ int launch_any(const GemmArgs& a, int tile_cfg, int grid, hipStream_t s)
 {
     switch (tile_cfg) {
         case 1: return launch_cfg<128, 128, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
-        case 3: return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
-        case 5: return launch_cfg<256, 256, 4, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+        case 3:
+            // four waves with 256 accumulator registers each leave the gated-backward epilogue no
+            // room for its operands: that shape is not built for it
+            if constexpr (EPI == EPI_GATED_BWD) {
+                amoe_set_error("grouped_gemm: tile_cfg 3 is not available with the gated-backward epilogue");
+                return AMOE_ERR_UNSUPPORTED;
+            } else {
+                return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+            }
+        case 5:
+            if constexpr (EPI == EPI_GATED_BWD) {   // spills as well (four tile columns per wave)
+                amoe_set_error("grouped_gemm: tile_cfg 5 is not available with the gated-backward epilogue");
+                return AMOE_ERR_UNSUPPORTED;
+            } else {
+                return launch_cfg<256, 256, 4, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+            }
         case 2: return launch_cfg<256, 128, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
         default: return launch_cfg<256, 256, 2, 4, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);  // 8 waves, 128x64 per wave
     }
@@ -768,7 +896,7 @@ int amoe_build_tile_map(const int32_t* offsets, int R, int E, int bm, void* work
 template <bool B_KC, int EPI, int ACT>
 static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C,
                          void* C2, const float* row_scale, int R, int E, int Kred, int N, int ldb, long long strideB, void* workspace,
-                         size_t workspace_bytes, int tile_cfg, hipStream_t s)
+                         size_t workspace_bytes, int tile_cfg, hipStream_t s, const void* G = nullptr, float* partials = nullptr)
 {
     const bool map_ready = (tile_cfg & AMOE_TILE_MAP_READY) != 0;
     tile_cfg &= ~AMOE_TILE_MAP_READY;
@@ -787,8 +915,12 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
     a.offsets = offsets;
     a.lda = Kred;
     a.ldb = ldb;
-    a.ldc = N;
+    a.ldc = EPI == EPI_GATED_BWD ? 2 * N : N;
     a.ldc2 = N / 2;
+    a.G = (const bf16_t*)G;
+    a.ldg = 2 * N;
+    a.partials = partials;
+    a.part_stride = R;
     a.strideB = strideB;
     a.strideC = 0;
     a.E = E;
@@ -827,6 +959,27 @@ int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const i
 {
     return run_rows_bf16<true, EPI_STORE, 0>(A, a_row_map, B, offsets, C, nullptr, nullptr, R, E, /*Kred=*/N, /*N out=*/Kd,
                                              /*ldb=*/N, (long long)Kd * N, workspace, workspace_bytes, tile_cfg, s);
+}
+
+// d_gate_up [R, 2I] and the row sums of the score gradient from dy rows [., H], w_down [E, I, H] and the
+// forward's gate_up [R, 2I]: the data gradient of the down projection with the backward of the gated
+// activation as its epilogue.  The reduction runs over H, the output columns are the I intermediate columns.
+int amoe_bf16_nt_gated_bwd(const void* dy, const int32_t* a_row_map, const void* w_down, const int32_t* offsets,
+                           const void* gate_up, const float* row_scale, void* d_gate_up, float* partials, int R, int E,
+                           int I, int H, int act, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s)
+{
+    AMOE_DISPATCH_ACT(act, return (run_rows_bf16<true, EPI_GATED_BWD, ACT>(dy, a_row_map, w_down, offsets, d_gate_up, nullptr,
+                                                                           row_scale, R, E, /*Kred=*/H, /*N out=*/I, /*ldb=*/H,
+                                                                           (long long)I * H, workspace, workspace_bytes,
+                                                                           tile_cfg, s, gate_up, partials)))
+    return AMOE_ERR_BAD_ARG;
+}
+
+// number of row-sum partials per routed row that amoe_bf16_nt_gated_bwd writes: one per N tile
+int amoe_bf16_gated_bwd_parts(int I, int tile_cfg)
+{
+    TileCfg tc = pick_cfg(tile_cfg & ~AMOE_TILE_MAP_READY);
+    return (I + tc.bn - 1) / tc.bn;
 }
 
 int amoe_bf16_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,

@@ -180,6 +180,19 @@ gated_act_bwd_kernel(const T* __restrict__ gu, const T* __restrict__ d_inter, co
     }
 }
 
+// d_scores[t,k] = sum_p partials[p][row_of[t,k]]  (fixed order over p)
+__global__ void __launch_bounds__(kBlock)
+score_grad_gather_kernel(const float* __restrict__ partials, int n_parts, long long part_stride,
+                         const int32_t* __restrict__ row_of, float* __restrict__ d_scores, int n_slots)
+{
+    const int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= n_slots) return;
+    const int row = row_of[s];
+    float tot = 0.f;
+    for (int p = 0; p < n_parts; ++p) tot += partials[p * part_stride + row];
+    d_scores[s] = tot;
+}
+
 int check_rows(const char* what, int dtype, int rows, int H)
 {
     AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "%s: bad dtype %d", what, dtype);
@@ -318,4 +331,16 @@ AMOE_EXPORT int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, con
                                (const float*)d_inter, row_scale, slot_of, T, K, (float*)d_gate_up, d_row_scale, R, I);
     })
     return amoe_check_launch("gated_act_bwd");
+}
+
+AMOE_EXPORT int amoe_score_grad_gather(const float* partials, int n_parts, const int32_t* row_of, float* d_scores, int T,
+                                       int K, void* stream)
+{
+    AMOE_REQUIRE(partials && row_of && d_scores, AMOE_ERR_BAD_ARG, "score_grad_gather: null pointer");
+    AMOE_REQUIRE(n_parts > 0 && T > 0 && K > 0, AMOE_ERR_BAD_ARG, "score_grad_gather: sizes must be positive");
+    AMOE_REQUIRE((long long)T * K < (1ll << 31), AMOE_ERR_UNSUPPORTED, "score_grad_gather: T*K does not fit int32");
+    const int n = T * K;
+    hipLaunchKernelGGL(score_grad_gather_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream,
+                       partials, n_parts, (long long)n, row_of, d_scores, n);
+    return amoe_check_launch("score_grad_gather");
 }

@@ -259,15 +259,28 @@ class _ExpertLayerFn(torch.autograd.Function):
 
         # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMMs' loads
         ws = ctx.gemm_ws  # still holds the forward's tile map
-        d_inter_s = ops.grouped_gemm_nt(dy, w_down, offsets, a_row_map=token_of, n_rows=R, tile_cfg=cfg, workspace=ws,
-                                        map_ready=True)
+        fused = x.dtype == torch.bfloat16 and cfg in (0, 1, 2)
+        if fused:
+            # data gradient of the down projection with the gated-activation backward as its
+            # epilogue: d_inter is never written; the score gradients come back as per-N-tile row sums
+            d_gate_up, parts = ops.grouped_gemm_nt_gated_bwd(
+                dy, w_down, offsets, gate_up, opts["act"], row_scale=scores_perm, a_row_map=token_of, n_rows=R, tile_cfg=cfg,
+                workspace=ws, map_ready=True,
+            )
+            if ds_perm is not None:  # gradient of the returned scores [R] (row order): one more partial
+                parts = torch.cat((parts, ds_perm.float().reshape(1, R)))
+                ds_perm = None
+            d_scores = ops.score_grad_gather(parts, row_of)
+        else:
+            d_inter_s = ops.grouped_gemm_nt(dy, w_down, offsets, a_row_map=token_of, n_rows=R, tile_cfg=cfg, workspace=ws,
+                                            map_ready=True)
+            # gated-activation backward, with the score multiply: also yields d_scores [T,K]
+            d_gate_up, d_scores = ops.gated_act_bwd(
+                gate_up, d_inter_s, opts["act"], row_scale=scores_perm, slot_of=slot_of, tk=(T, K)
+            )
         d_w_down = None
         if ctx.needs_input_grad[3]:
             d_w_down = ops.grouped_gemm_wgrad(inter_s, dy, offsets, E, tile_cfg=cfg, b_row_map=token_of)
-        # gated-activation backward, with the score multiply: also yields d_scores [T,K]
-        d_gate_up, d_scores = ops.gated_act_bwd(
-            gate_up, d_inter_s, opts["act"], row_scale=scores_perm, slot_of=slot_of, tk=(T, K)
-        )
         d_w_gate_up = None
         if ctx.needs_input_grad[2]:
             d_w_gate_up = ops.grouped_gemm_wgrad(x, d_gate_up, offsets, E, tile_cfg=cfg, a_row_map=token_of)

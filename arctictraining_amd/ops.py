@@ -279,6 +279,52 @@ def grouped_gemm_nt(A, B, offsets, a_row_map=None, n_rows=None, tile_cfg: int = 
     return C
 
 
+def grouped_gemm_nt_gated_bwd(dy, w_down, offsets, gate_up, act: int = ACT_SILU, row_scale=None, a_row_map=None,
+                              n_rows=None, want_score_parts: bool = True, tile_cfg: int = 0, workspace=None,
+                              map_ready: bool = False):
+    """d_gate_up [R,2I] and score partials [n_parts,R] f32 (None unless wanted) from dy rows [.,H]
+    (gathered through a_row_map), w_down [E,I,H] and the forward's gate_up [R,2I]: the data gradient
+    of the down projection with the gated-activation backward as its epilogue (bf16 only)."""
+    lib = _lib.load()
+    _chk(dy, "dy", torch.bfloat16)
+    _chk(w_down, "w_down", torch.bfloat16)
+    _chk(gate_up, "gate_up", torch.bfloat16)
+    _chk(offsets, "offsets", torch.int32)
+    if a_row_map is not None:
+        _chk(a_row_map, "a_row_map", torch.int32)
+    if row_scale is not None:
+        _chk(row_scale, "row_scale", torch.float32)
+    E, I, H = w_down.shape
+    R = int(n_rows if n_rows is not None else (a_row_map.numel() if a_row_map is not None else dy.shape[0]))
+    if gate_up.shape != (R, 2 * I):
+        raise RuntimeError(f"gate_up must be [{R}, {2 * I}], got {tuple(gate_up.shape)}")
+    d_gate_up = torch.empty_like(gate_up)
+    parts = None
+    if want_score_parts:
+        parts = torch.empty((lib.amoe_gated_bwd_score_parts(I, tile_cfg), R), dtype=torch.float32, device=dy.device)
+    ws, tile_cfg = _ws_and_cfg(R, E, dy.device, tile_cfg, workspace, map_ready)
+    rc = lib.amoe_grouped_gemm_nt_gated_bwd(
+        dy.data_ptr(), _ptr(a_row_map), w_down.data_ptr(), offsets.data_ptr(), gate_up.data_ptr(), _ptr(row_scale),
+        d_gate_up.data_ptr(), _ptr(parts), BF16, R, E, I, H, act, ws.data_ptr(), ws.numel(), tile_cfg, _stream()
+    )
+    _lib.check(rc, "amoe_grouped_gemm_nt_gated_bwd")
+    return d_gate_up, parts
+
+
+def score_grad_gather(parts: torch.Tensor, row_of: torch.Tensor) -> torch.Tensor:
+    """d_scores [T,K] f32 = sum over the partials [n_parts, T*K] of the entry at row_of[t,k]."""
+    lib = _lib.load()
+    _chk(parts, "parts", torch.float32)
+    _chk(row_of, "row_of", torch.int32)
+    T, K = row_of.shape
+    if parts.dim() != 2 or parts.shape[1] != T * K:
+        raise RuntimeError(f"parts must be [n_parts, {T * K}], got {tuple(parts.shape)}")
+    d_scores = torch.empty((T, K), dtype=torch.float32, device=parts.device)
+    rc = lib.amoe_score_grad_gather(parts.data_ptr(), parts.shape[0], row_of.data_ptr(), d_scores.data_ptr(), T, K, _stream())
+    _lib.check(rc, "amoe_score_grad_gather")
+    return d_scores
+
+
 def grouped_gemm_wgrad(A, B, offsets, num_experts: int, tile_cfg: int = 0, a_row_map=None, b_row_map=None) -> torch.Tensor:
     """C[e] = A[rows_e,:]^T @ B[rows_e,:];  A [R,Kd], B [R,N] -> C [E,Kd,N].  With a_row_map [R] (or
     b_row_map [R]) the rows of A (or B) are gathered from a smaller matrix inside the kernel."""

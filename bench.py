@@ -11,8 +11,8 @@ a bounded sample of the same workload as a baseline.
 
 c4 is one expert-parallel rank's share of a DeepSeek-V3-like layer: 65536 routed rows that
 arrive already assigned to 32 local experts (Zipf(1.2) loads), so there is no router; its
-step is the grouped expert FFN forward + backward (six grouped GEMMs and the gated
-activation backward) and its throughput is counted in routed rows.
+step is the grouped expert FFN forward + backward (six grouped GEMMs, the gated activation
+backward being the epilogue of one of them) and its throughput is counted in routed rows.
 """
 import argparse
 import json
@@ -202,9 +202,13 @@ def main():
             ws = ops.gemm_workspace(R, E, dev)
             gu_, in_ = ops.grouped_gemm_gateup_act_fwd(xd, wgu_d, offsets, row_scale=s_perm, tile_cfg=c, workspace=ws)
             ops.grouped_gemm_nn(in_, wd_d, offsets, tile_cfg=c, workspace=ws, map_ready=True)
-            di_ = ops.grouped_gemm_nt(dyg, wd_d, offsets, tile_cfg=c, workspace=ws, map_ready=True)
+            if c in (0, 1, 2):
+                dg_, _ = ops.grouped_gemm_nt_gated_bwd(dyg, wd_d, offsets, gu_, row_scale=s_perm, tile_cfg=c, workspace=ws,
+                                                       map_ready=True)
+            else:
+                di_ = ops.grouped_gemm_nt(dyg, wd_d, offsets, tile_cfg=c, workspace=ws, map_ready=True)
+                dg_ = ops.gated_act_bwd(gu_, di_, row_scale=s_perm)
             ops.grouped_gemm_wgrad(in_, dyg, offsets, E, tile_cfg=c)
-            dg_ = ops.gated_act_bwd(gu_, di_, row_scale=s_perm)
             ops.grouped_gemm_wgrad(xd, dg_, offsets, E, tile_cfg=c)
             ops.grouped_gemm_nt(dg_, wgu_d, offsets, tile_cfg=c, workspace=ws, map_ready=True)
 
@@ -265,6 +269,7 @@ def main():
     d_inter = ops.grouped_gemm_nt(dyg, wd_d, offsets, a_row_map=token_of, n_rows=R, tile_cfg=c)
     d_gu = ops.gated_act_bwd(gu, d_inter)
     d_xp = ops.grouped_gemm_nt(d_gu, wgu_d, offsets, tile_cfg=c)
+    fused_bwd = dtype == torch.bfloat16 and c in (0, 1, 2)   # what the layer's backward does
     # the kernel symbol (template instance) each launch resolves to: what rocprofv3 reports
     tile = {1: "128, 128, 2, 2", 2: "256, 128, 2, 2", 3: "256, 256, 2, 2", 5: "256, 256, 4, 2"}.get(c, "256, 256, 2, 4")
     gathered = token_of is not None
@@ -272,6 +277,7 @@ def main():
         "gemm_gateup_act_fwd": f"grouped_gemm_bf16_kernel<{tile}, true, false, 1, 0, 0>",
         "gemm_down_fwd": f"grouped_gemm_bf16_kernel<{tile}, true, false, 0, 0, 0>",
         "gemm_dgrad_down": f"grouped_gemm_bf16_kernel<{tile}, true, true, 0, 0, 0>",
+        "gemm_dgrad_down_gated_bwd": f"grouped_gemm_bf16_kernel<{tile}, true, true, 2, 0, 0>",
         "gemm_dgrad_gateup": f"grouped_gemm_bf16_kernel<{tile}, true, true, 0, 0, 0>",
         "gemm_wgrad_down": f"grouped_gemm_bf16_kernel<{tile}, false, false, 0, 0, {2 if gathered else 0}>",
         "gemm_wgrad_gateup": f"grouped_gemm_bf16_kernel<{tile}, false, false, 0, 0, {1 if gathered else 0}>",
@@ -281,7 +287,8 @@ def main():
     # dense equivalents (M, K, N, layout) of the grouped launches, for the library yardstick
     dense = {
         "gemm_gateup_act_fwd": (R, H, 2 * I, "nn"), "gemm_down_fwd": (R, I, H, "nn"),
-        "gemm_dgrad_down": (R, H, I, "nt"), "gemm_dgrad_gateup": (R, 2 * I, H, "nt"),
+        "gemm_dgrad_down": (R, H, I, "nt"), "gemm_dgrad_down_gated_bwd": (R, H, I, "nt"),
+        "gemm_dgrad_gateup": (R, 2 * I, H, "nt"),
         "gemm_wgrad_down": (I, R, H, "tn"), "gemm_wgrad_gateup": (H, R, 2 * I, "tn"),
     }
     # (name, callable, flops per launch, algorithmic bytes per launch)
@@ -291,6 +298,12 @@ def main():
          (A_T * H + E * H * 2 * I + 3 * R * I) * es),
         ("gemm_down_fwd", lambda: ops.grouped_gemm_nn(inter, wd_d, offsets, tile_cfg=c), 2.0 * R * H * I,
          (R * I + E * I * H + R * H) * es),
+        # bf16: the data gradient of the down projection carries the gated-activation backward as its
+        # epilogue (reads gate_up, writes d_gate_up and the score-gradient partials; d_inter is never stored)
+        ("gemm_dgrad_down_gated_bwd", lambda: ops.grouped_gemm_nt_gated_bwd(dyg, wd_d, offsets, gu, row_scale=s_perm,
+                                                                            a_row_map=token_of, n_rows=R, tile_cfg=c),
+         2.0 * R * H * I, (A_T * H + E * I * H + 4 * R * I) * es + 4 * R * ((I + 255) // 256))
+        if fused_bwd else
         ("gemm_dgrad_down", lambda: ops.grouped_gemm_nt(dyg, wd_d, offsets, a_row_map=token_of, n_rows=R, tile_cfg=c),
          2.0 * R * H * I, (A_T * H + E * I * H + R * I) * es),
         ("gemm_wgrad_down", lambda: ops.grouped_gemm_wgrad(inter, dyg, offsets, E, tile_cfg=c, b_row_map=token_of),
@@ -299,13 +312,20 @@ def main():
          (2 * R * I + E * H * 2 * I + R * H) * es),
         ("gemm_wgrad_gateup", lambda: ops.grouped_gemm_wgrad(xd, d_gu, offsets, E, tile_cfg=c, a_row_map=token_of),
          4.0 * R * H * I, (A_T * H + 2 * R * I + E * H * 2 * I) * es),
-        ("gated_act_bwd", lambda: ops.gated_act_bwd(gu, d_inter, row_scale=s_perm), 0.0, 5 * R * I * es + 4 * R),
     ]
+    if not fused_bwd:
+        kernels.append(("gated_act_bwd", lambda: ops.gated_act_bwd(gu, d_inter, row_scale=s_perm), 0.0, 5 * R * I * es + 4 * R))
     if name != "c4":
         probs, topk_idx, counts_d = cap["probs"], cap["topk_idx"], cap["counts"]
         d_scores = cap["d_scores"]
-        kernels[-1] = ("gated_act_bwd", lambda: ops.gated_act_bwd(gu, d_inter, row_scale=s_perm, slot_of=slot_of, tk=(T, K)),
-                       0.0, 5 * R * I * es + 12 * R)
+        if fused_bwd:
+            parts = ops.grouped_gemm_nt_gated_bwd(dyg, wd_d, offsets, gu, row_scale=s_perm, a_row_map=token_of, n_rows=R,
+                                                  tile_cfg=c)[1]
+            kernels.append(("score_grad_gather", lambda: ops.score_grad_gather(parts, row_of), 0.0,
+                            (parts.shape[0] + 2) * R * 4))
+        else:
+            kernels[-1] = ("gated_act_bwd", lambda: ops.gated_act_bwd(gu, d_inter, row_scale=s_perm, slot_of=slot_of, tk=(T, K)),
+                           0.0, 5 * R * I * es + 12 * R)
         kernels += [
             ("combine_fwd", lambda: ops.combine_fwd(out, row_of, None), 0.0, (R + T) * H * es + R * 4),
             ("gather_rows_bwd", lambda: ops.gather_rows_bwd(d_xp, row_of, None), 0.0, (R + T) * H * es),

@@ -183,6 +183,37 @@ int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, const void* B,
                          int tile_cfg, void* stream);
 
 /*
+ * Data gradient of the down projection with the backward of the gated activation as its
+ * epilogue (autograd of moe.py:187-192 through moe.py:59, plus the score gradient that the
+ * reference takes in the backward of moe.py:460): d_inter = dy_rows @ w_down[e]^T is formed in
+ * registers and never stored;
+ *   d_gate_up[r,2i]   = row_scale[r] * d_inter[r,i] * up * act'(gate)
+ *   d_gate_up[r,2i+1] = row_scale[r] * d_inter[r,i] * act(gate)          (gate, up) = gate_up[r,2i..2i+1]
+ *   score_partials[p][r] = sum over the i of N tile p of d_inter[r,i] * up * act(gate)
+ * dy [., H] (rows gathered through a_row_map when non-null), w_down [E,I,H], gate_up [R,2I] of
+ * the forward pass, row_scale [R] f32 or null (= 1), d_gate_up [R,2I].  score_partials is
+ * [amoe_gated_bwd_score_parts(I, tile_cfg)][R] f32 or null; summing it over p gives the gradient
+ * of row_scale[r] (amoe_score_grad_gather does that and takes the rows back to their slots).
+ * bf16 only, tile_cfg 0, 1 or 2 (AMOE_ERR_UNSUPPORTED otherwise: such callers run
+ * amoe_grouped_gemm_nt and amoe_gated_act_bwd).  Same result as those two calls up to the rounding of d_inter to the
+ * model dtype, which this path skips.
+ */
+int amoe_gated_bwd_score_parts(int I, int tile_cfg);
+int amoe_grouped_gemm_nt_gated_bwd(const void* dy, const int32_t* a_row_map, const void* w_down, const int32_t* offsets,
+                                   const void* gate_up, const float* row_scale, void* d_gate_up, float* score_partials,
+                                   int dtype, int R, int E, int I, int H, int act, void* workspace, size_t workspace_bytes,
+                                   int tile_cfg, void* stream);
+
+/*
+ * d_scores[t,k] = sum_p score_partials[p][row_of[t,k]]: the row sums of
+ * amoe_grouped_gemm_nt_gated_bwd (score_partials [n_parts][T*K]) added up in a fixed order and
+ * taken from routed-row order back to the slots [T,K] (the scatter that autograd performs for
+ * topk_scores[token_mapped_slots], moe.py:379).
+ */
+int amoe_score_grad_gather(const float* score_partials, int n_parts, const int32_t* row_of, float* d_scores, int T, int K,
+                           void* stream);
+
+/*
  * Grouped weight-gradient GEMM:  C[e] = A[rows_e,:]^T @ B[rows_e,:]   (zeros for an empty
  * expert).  A [R,Kd], B [R,N], C [E,Kd,N].  The autograd of moe.py:59 w.r.t. B[e].
  * One of the operands may be gathered: with a_row_map [R], row r of A is read from

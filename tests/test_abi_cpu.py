@@ -114,6 +114,21 @@ def test_gemm_argument_errors(lib):
     assert lib.amoe_grouped_gemm_gateup_act_fwd(P, None, P, P, None, None, P, 0, 128, 4, 64, 64, 0, P, big, 0, None) == -2
 
 
+def test_gated_bwd_gemm_argument_errors(lib):
+    big = 1 << 20
+    f = lib.amoe_grouped_gemm_nt_gated_bwd
+    assert f(P, None, P, P, None, None, P, None, 1, 128, 4, 64, 64, 0, P, big, 0, None) == -1  # gate_up is required
+    assert f(P, None, P, P, P, None, P, None, 0, 128, 4, 64, 64, 0, P, big, 0, None) == -2  # float32
+    assert b"bf16 only" in lib.amoe_last_error()
+    assert f(P, None, P, P, P, None, P, None, 1, 128, 4, 64, 48, 0, P, big, 0, None) == -2  # H not a multiple of 32
+    assert f(P, None, P, P, P, None, P, None, 1, 128, 4, 64, 64, 9, P, big, 0, None) == -1  # activation
+    assert f(P, None, P, P, P, None, P, None, 1, 128, 4, 64, 64, 0, P, 8, 0, None) == -3  # workspace
+    assert lib.amoe_gated_bwd_score_parts(768, 0) == 3 and lib.amoe_gated_bwd_score_parts(768, 1) == 6
+    assert lib.amoe_gated_bwd_score_parts(0, 0) == 0
+    assert lib.amoe_score_grad_gather(None, 3, P, P, 4, 2, None) == -1
+    assert lib.amoe_score_grad_gather(P, 0, P, P, 4, 2, None) == -1
+
+
 def test_remap_argument_errors(lib):
     assert lib.amoe_remap_pack(None, P, P, 1, 2, 64, 64, 64 * 64, None) == -1
     assert lib.amoe_remap_pack(P, P, P, 5, 2, 64, 64, 64 * 64, None) == -1  # dtype

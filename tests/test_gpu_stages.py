@@ -383,6 +383,64 @@ def test_gateup_activation_fused(ops, gpu_device, dtype, cfg, act):
     assert O.rel_l2(inter3.cpu(), ref_inter * rs.double()[:, None]) <= (BF16_TOL if dtype == torch.bfloat16 else 2e-5)
 
 
+@pytest.mark.parametrize("cfg", [0, 1, 2])
+@pytest.mark.parametrize("act", ["silu", "gpt_oss", "gelu"])
+def test_dgrad_down_with_gated_activation_backward(ops, gpu_device, cfg, act):
+    """The data gradient of the down projection with the gated-activation backward as its epilogue
+    (autograd of moe.py:187-192 and of the score multiply of moe.py:460): d_gate_up and the score
+    gradients against float64 autograd over the same rounded inputs, and against the two-kernel
+    path it replaces."""
+    _say("dgrad_down+gated_bwd", cfg, act)
+    code = {"silu": 0, "gelu": 1, "relu": 2, "gpt_oss": 3}[act]
+    g = torch.Generator().manual_seed(23)
+    T, K, E, H, I = 230, 4, 6, 128, 352          # I: two N tiles of 256 (the second ragged), or three of 128
+    R = T * K
+    assign = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    assign[assign == 2] = 3                       # an empty expert
+    perm, tok, counts = O.permutation(assign, E)
+    offs = _offsets(counts, gpu_device)
+    row_of = O.inverse_row_map(perm, T, K).to(torch.int32).to(gpu_device)
+    bf = torch.bfloat16
+    dy = torch.randn(T, H, generator=g).to(bf)
+    wd = (torch.randn(E, I, H, generator=g) * 0.1).to(bf)
+    gu = torch.randn(R, 2 * I, generator=g).to(bf)
+    s_perm = torch.rand(R, generator=g) + 0.1
+    d = gpu_device
+    d_gu, parts = ops.grouped_gemm_nt_gated_bwd(dy.to(d), wd.to(d), offs, gu.to(d), code, row_scale=s_perm.to(d),
+                                                a_row_map=tok.to(torch.int32).to(d), n_rows=R, tile_cfg=cfg)
+    d_s = ops.score_grad_gather(parts, row_of)
+    torch.cuda.synchronize()
+    # float64 autograd of inter_s = s * up * act(gate), out = inter_s @ W_down[e], loss = <dy[tok], out>
+    gu64 = gu.double().requires_grad_(True)
+    s64 = s_perm.double().requires_grad_(True)
+    inter = s64[:, None] * gu64[:, 1::2] * O.activation(act)(gu64[:, 0::2])
+    out = O.grouped_gemm(inter, wd.double(), counts.cumsum(0))
+    (out * dy.double()[tok]).sum().backward()
+    assert O.rel_l2(d_gu.cpu(), gu64.grad) <= 5e-3, "d_gate_up"
+    ref_ds = torch.zeros(R, dtype=torch.float64)
+    ref_ds[perm] = s64.grad
+    assert O.rel_l2(d_s.cpu(), ref_ds.view(K, T).t()) <= 5e-3, "score gradients"
+    # the two kernels it replaces (they round d_inter to bf16 in between)
+    d_inter = ops.grouped_gemm_nt(dy.to(d), wd.to(d), offs, a_row_map=tok.to(torch.int32).to(d), n_rows=R, tile_cfg=cfg)
+    d_gu2, d_s2 = ops.gated_act_bwd(gu.to(d), d_inter, code, row_scale=s_perm.to(d),
+                                    slot_of=perm.to(torch.int32).to(d), tk=(T, K))
+    assert O.rel_l2(d_gu.cpu(), d_gu2.cpu().double()) <= 5e-3
+    assert O.rel_l2(d_s.cpu(), d_s2.cpu().double()) <= 5e-3
+    # without the partials, and without a row scale
+    d_gu3, none = ops.grouped_gemm_nt_gated_bwd(dy.to(d), wd.to(d), offs, gu.to(d), code, row_scale=s_perm.to(d),
+                                                a_row_map=tok.to(torch.int32).to(d), n_rows=R, tile_cfg=cfg,
+                                                want_score_parts=False)
+    assert none is None and torch.equal(d_gu3, d_gu)
+    d_gu4, _ = ops.grouped_gemm_nt_gated_bwd(dy.to(d)[tok.to(d)].contiguous(), wd.to(d), offs, gu.to(d), code, tile_cfg=cfg)
+    gu64b = gu.double().requires_grad_(True)
+    inter = gu64b[:, 1::2] * O.activation(act)(gu64b[:, 0::2])
+    (O.grouped_gemm(inter, wd.double(), counts.cumsum(0)) * dy.double()[tok]).sum().backward()
+    assert O.rel_l2(d_gu4.cpu(), gu64b.grad) <= 5e-3
+    with pytest.raises(RuntimeError, match="tile_cfg 3"):
+        ops.grouped_gemm_nt_gated_bwd(dy.to(d), wd.to(d), offs, gu.to(d), code, a_row_map=tok.to(torch.int32).to(d),
+                                      n_rows=R, tile_cfg=3)
+
+
 def test_grouped_gemm_rows_outside_groups_untouched(ops, gpu_device):
     """Rows past offsets[E] are never written (the tile map covers only routed rows)."""
     g = torch.Generator().manual_seed(5)
