@@ -30,6 +30,11 @@ SIGNATURES = {
         [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
          _c_void_p, _c_size_t, _c_void_p],
     ),
+    "amoe_permute_plan_tiled": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+         _c_void_p, _c_size_t, _c_void_p, _c_size_t, _c_int, _c_int, _c_void_p],
+    ),
     "amoe_permute_plan_static": (
         _c_int,
         [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,

@@ -892,6 +892,24 @@ int amoe_build_tile_map(const int32_t* offsets, int R, int E, int bm, void* work
     return amoe_check_launch("tile_map");
 }
 
+// Where the tile map of a row-grouped GEMM lives inside its workspace and how tall its tiles are, for a
+// caller that builds the map itself (the permutation plan): the float32 kernels use 64-row tiles.
+int amoe_tile_map_layout(int R, int E, int dtype, int tile_cfg, void* workspace, size_t workspace_bytes, int4** tile_map,
+                         int32_t** n_mtiles, int* bm, int* max_mtiles)
+{
+    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "tile map: bad dtype %d", dtype);
+    const int shape = tile_cfg & ~AMOE_TILE_MAP_READY;
+    AMOE_REQUIRE(tile_cfg >= 0 && shape <= 5 && shape != 4, AMOE_ERR_BAD_ARG, "tile map: bad tile_cfg %d", tile_cfg);
+    AMOE_REQUIRE(R > 0 && E > 0 && E <= AMOE_MAX_EXPERTS, AMOE_ERR_BAD_ARG, "tile map: bad sizes R=%d E=%d", R, E);
+    AMOE_REQUIRE(workspace_bytes >= amoe_grouped_gemm_workspace_bytes(R, E), AMOE_ERR_WORKSPACE,
+                 "tile map: workspace %zu < %zu bytes", workspace_bytes, amoe_grouped_gemm_workspace_bytes(R, E));
+    *bm = dtype == AMOE_F32 ? 64 : pick_cfg(shape).bm;
+    *max_mtiles = ws_max_mtiles(R, E, *bm);
+    *n_mtiles = (int32_t*)workspace;
+    *tile_map = (int4*)((char*)workspace + 16);
+    return AMOE_OK;
+}
+
 // rows mode driver shared by the three row-grouped entry points
 template <bool B_KC, int EPI, int ACT>
 static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C,

@@ -44,15 +44,23 @@ permute_hist_kernel(const int32_t* __restrict__ assign, int T, int K, int E, int
 
 // One block of 1024 threads: with EP = E rounded up to a power of two, thread t works for
 // expert t % EP on the (t / EP)-th slice of the chunks, so that the walk over chunks (the only
-// sequential part) is 1024 / EP ways parallel and every load is coalesced over experts.
+// sequential part) is 1024 / EP ways parallel and every load is coalesced over experts.  A
+// thread holds its slice of counts in registers between the two passes (kScanBatch at a time):
+// the exclusive bases overwrite the counts in place, and loads issued after such a store cannot
+// be moved ahead of it, which would turn the second pass into a chain of dependent round trips.
+// When tile_map is non-null the block also writes the row-grouped GEMMs' tile map (one int4
+// {expert, first row, end row, 0} per `bm`-row tile, {-1,0,0,0} past the last) and its tile count.
 constexpr int kScanThreads = 1024;
+constexpr int kScanBatch = 16;
 
 __global__ void __launch_bounds__(kScanThreads)
 permute_scan_kernel(int32_t* __restrict__ chunk_counts /* in: counts, out: exclusive base inside expert */,
-                    int E, int EP, int n_chunks, int32_t* __restrict__ counts, int32_t* __restrict__ offsets)
+                    int E, int EP, int n_chunks, int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+                    int4* __restrict__ tile_map, int32_t* __restrict__ n_mtiles, int bm, int max_mtiles)
 {
     __shared__ int32_t part[kScanThreads];       // [slice][EP]
-    __shared__ int32_t tot[AMOE_MAX_EXPERTS];
+    __shared__ int32_t tot[AMOE_MAX_EXPERTS + 1];
+    __shared__ int32_t tstart[AMOE_MAX_EXPERTS + 1];
     const int t = threadIdx.x;
     const int e = t & (EP - 1);
     const int g = t / EP;
@@ -61,7 +69,13 @@ permute_scan_kernel(int32_t* __restrict__ chunk_counts /* in: counts, out: exclu
     const int c0 = min(g * per, n_chunks), c1 = min(c0 + per, n_chunks);
     int sum = 0;
     if (e < E)
-        for (int c = c0; c < c1; ++c) sum += chunk_counts[(size_t)c * E + e];
+        for (int cb = c0; cb < c1; cb += kScanBatch) {
+            int v[kScanBatch];
+#pragma unroll
+            for (int i = 0; i < kScanBatch; ++i) v[i] = cb + i < c1 ? chunk_counts[(size_t)(cb + i) * E + e] : 0;
+#pragma unroll
+            for (int i = 0; i < kScanBatch; ++i) sum += v[i];
+        }
     part[t] = sum;
     __syncthreads();
     int run = 0;
@@ -71,22 +85,69 @@ permute_scan_kernel(int32_t* __restrict__ chunk_counts /* in: counts, out: exclu
         tot[e] = run + sum;
     }
     if (e < E)
-        for (int c = c0; c < c1; ++c) {
-            int v = chunk_counts[(size_t)c * E + e];
-            chunk_counts[(size_t)c * E + e] = run;
-            run += v;
+        for (int cb = c0; cb < c1; cb += kScanBatch) {
+            int v[kScanBatch];
+#pragma unroll
+            for (int i = 0; i < kScanBatch; ++i) v[i] = cb + i < c1 ? chunk_counts[(size_t)(cb + i) * E + e] : 0;
+#pragma unroll
+            for (int i = 0; i < kScanBatch; ++i) {
+                if (cb + i < c1) chunk_counts[(size_t)(cb + i) * E + e] = run;
+                run += v[i];
+            }
         }
     if (t < AMOE_MAX_EXPERTS && t >= E) tot[t] = 0;
     __syncthreads();
-    // Hillis-Steele inclusive scan over experts
-    for (int o = 1; o < AMOE_MAX_EXPERTS; o <<= 1) {
-        int add = (t < AMOE_MAX_EXPERTS && t >= o) ? tot[t - o] : 0;
-        __syncthreads();
-        if (t < AMOE_MAX_EXPERTS) tot[t] += add;
-        __syncthreads();
+    // Inclusive scans over the experts of the row counts and of the per-expert tile counts, by ONE
+    // wavefront: 8 consecutive entries per lane serially, the lane sums by cross-lane shuffles
+    // (a block-wide Hillis-Steele scan costs 18 barriers of 16 wavefronts).
+    static_assert(AMOE_MAX_EXPERTS == 8 * AMOE_WAVE, "one wavefront scans 8 entries per lane");
+    if (t < AMOE_WAVE) {
+        int r[8], rt[8];
+        int s_rows = 0, s_tiles = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            r[i] = tot[t * 8 + i];
+            rt[i] = (r[i] + bm - 1) / bm;
+            s_rows += r[i];
+            s_tiles += rt[i];
+        }
+        int in_rows = s_rows, in_tiles = s_tiles;
+#pragma unroll
+        for (int o = 1; o < AMOE_WAVE; o <<= 1) {
+            const int u = __shfl_up(in_rows, o, AMOE_WAVE), ut = __shfl_up(in_tiles, o, AMOE_WAVE);
+            if (t >= o) {
+                in_rows += u;
+                in_tiles += ut;
+            }
+        }
+        int run_rows = in_rows - s_rows, run_tiles = in_tiles - s_tiles;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            run_rows += r[i];
+            run_tiles += rt[i];
+            tot[t * 8 + i] = run_rows;
+            tstart[t * 8 + i] = run_tiles;
+        }
     }
+    __syncthreads();
     if (t < E) offsets[t + 1] = tot[t];
     if (t == 0) offsets[0] = 0;
+    if (tile_map == nullptr) return;
+    // tot[e] = end row of expert e, tstart[e] = first tile of expert e + 1 (inclusive scans)
+    const int total = tstart[E - 1];
+    if (t == 0) *n_mtiles = total < max_mtiles ? total : max_mtiles;
+    for (int mt = t; mt < total && mt < max_mtiles; mt += kScanThreads) {
+        // smallest ex with tstart[ex] > mt: the expert that owns tile mt
+        int lo = 0, hi = E - 1;
+        while (lo < hi) {
+            int mid = (lo + hi) >> 1;
+            if (tstart[mid] > mt) hi = mid; else lo = mid + 1;
+        }
+        const int first_tile = lo ? tstart[lo - 1] : 0;
+        const int row0 = lo ? tot[lo - 1] : 0;
+        tile_map[mt] = make_int4(lo, row0 + (mt - first_tile) * bm, tot[lo], 0);
+    }
+    for (int mt = total + t; mt < max_mtiles; mt += kScanThreads) tile_map[mt] = make_int4(-1, 0, 0, 0);
 }
 
 __global__ void __launch_bounds__(kWavesPerBlock * AMOE_WAVE)
@@ -160,7 +221,8 @@ static int check_plan_args(const int32_t* assign, const float* scores, int T, in
 // written by the histogram kernel before it is read: nothing has to be cleared)
 static int launch_plan(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
                        int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of, float* scores_perm,
-                       int32_t* cc, hipStream_t s)
+                       int32_t* cc, hipStream_t s, int4* tile_map = nullptr, int32_t* n_mtiles = nullptr, int bm = 1,
+                       int max_mtiles = 0)
 {
     const int R = T * K;
     const int n_chunks = permute_chunks(R);
@@ -169,7 +231,8 @@ static int launch_plan(const int32_t* assign, const float* scores, int T, int K,
                        n_chunks, cc);
     int EP = 1;
     while (EP < E) EP <<= 1;
-    hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, cc, E, EP, n_chunks, counts, offsets);
+    hipLaunchKernelGGL(permute_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, cc, E, EP, n_chunks, counts, offsets,
+                       tile_map, n_mtiles, bm, max_mtiles);
     hipLaunchKernelGGL(permute_scatter_kernel, dim3(n_blocks), dim3(kWavesPerBlock * AMOE_WAVE), 0, s, assign, T, K, E,
                        R, n_chunks, cc, offsets, scores, token_of, slot_of, row_of, scores_perm);
     return amoe_check_launch("permute_plan");
@@ -186,6 +249,31 @@ AMOE_EXPORT int amoe_permute_plan(const int32_t* assign, const float* scores, in
                  "permute_plan: workspace %zu < %zu bytes", workspace_bytes, amoe_permute_workspace_bytes(T * K, E));
     return launch_plan(assign, scores, T, K, E, counts, offsets, token_of, slot_of, row_of, scores_perm,
                        (int32_t*)workspace, (hipStream_t)stream);
+}
+
+// The plan together with the tile map of the row-grouped GEMMs that will run over its offsets: the
+// scan kernel holds the offsets anyway, so the map costs no launch of its own.
+int amoe_tile_map_layout(int R, int E, int dtype, int tile_cfg, void* workspace, size_t workspace_bytes, int4** tile_map,
+                         int32_t** n_mtiles, int* bm, int* max_mtiles);
+
+AMOE_EXPORT int amoe_permute_plan_tiled(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                                        int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of,
+                                        float* scores_perm, void* workspace, size_t workspace_bytes, void* gemm_workspace,
+                                        size_t gemm_workspace_bytes, int dtype, int tile_cfg, void* stream)
+{
+    int rc = check_plan_args(assign, scores, T, K, E, counts, offsets, token_of, slot_of, row_of, scores_perm);
+    if (rc) return rc;
+    AMOE_REQUIRE(workspace && gemm_workspace, AMOE_ERR_BAD_ARG, "permute_plan_tiled: null workspace");
+    AMOE_REQUIRE(workspace_bytes >= amoe_permute_workspace_bytes(T * K, E), AMOE_ERR_WORKSPACE,
+                 "permute_plan_tiled: workspace %zu < %zu bytes", workspace_bytes, amoe_permute_workspace_bytes(T * K, E));
+    int4* tile_map = nullptr;
+    int32_t* n_mtiles = nullptr;
+    int bm = 0, max_mtiles = 0;
+    rc = amoe_tile_map_layout(T * K, E, dtype, tile_cfg, gemm_workspace, gemm_workspace_bytes, &tile_map, &n_mtiles, &bm,
+                              &max_mtiles);
+    if (rc) return rc;
+    return launch_plan(assign, scores, T, K, E, counts, offsets, token_of, slot_of, row_of, scores_perm,
+                       (int32_t*)workspace, (hipStream_t)stream, tile_map, n_mtiles, bm, max_mtiles);
 }
 
 // ------------------------------------------------------------------ the variant that allocates nothing

@@ -32,6 +32,50 @@ __device__ __forceinline__ unsigned long long row_lane_u64(unsigned long long k,
     return ((unsigned long long)hi << 32) | lo;
 }
 
+// The same order in 32 bits for bf16 logits: a bf16 value has 16 significant bits, so the upper
+// half of the monotone pattern decides, and the lower half is free for the index (E <= 512).
+// Half the instructions of the 64-bit key in every arg-max step.
+__device__ __forceinline__ uint32_t sel_key32(float v, int idx)
+{
+    v = v + 0.0f;
+    uint32_t u = __float_as_uint(v);
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    return (u & 0xffff0000u) | (0xffffu - (uint32_t)idx);
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t max_with_dpp(uint32_t k)
+{
+    const uint32_t other = dpp_u32<CTRL>(k);
+    return other > k ? other : k;
+}
+
+__device__ __forceinline__ uint32_t wave_max_key(uint32_t k)
+{
+    k = max_with_dpp<AMOE_DPP_QUAD_XOR1>(k);
+    k = max_with_dpp<AMOE_DPP_QUAD_XOR2>(k);
+    k = max_with_dpp<AMOE_DPP_HALF_MIRROR>(k);
+    k = max_with_dpp<AMOE_DPP_MIRROR>(k);
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)k, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)k, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)k, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)k, 48);
+    const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+
+// key type, construction and index extraction per logit type
+template <typename T>
+struct SelKey {
+    typedef unsigned long long type;
+    __device__ static __forceinline__ type make(float v, int idx) { return sel_key(v, idx); }
+    __device__ static __forceinline__ int index(type k) { return (int)(0xffffffffu - (uint32_t)(k & 0xffffffffull)); }
+};
+template <>
+struct SelKey<bf16_t> {
+    typedef uint32_t type;
+    __device__ static __forceinline__ type make(float v, int idx) { return sel_key32(v, idx); }
+    __device__ static __forceinline__ int index(type k) { return (int)(0xffffu - (k & 0xffffu)); }
+};
+
 // wave-uniform maximum of the 64 keys
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k)
 {
@@ -44,6 +88,7 @@ __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k)
     const unsigned long long ab = a > b ? a : b, cd = c > d ? c : d;
     return ab > cd ? ab : cd;
 }
+__device__ __forceinline__ unsigned long long wave_max_key(unsigned long long k) { return wave_max_u64(k); }
 
 template <typename T, int VPT>
 __global__ void __launch_bounds__(kTokensPerBlock * AMOE_WAVE)
@@ -55,14 +100,15 @@ router_topk_fwd_kernel(const T* __restrict__ logits, int n_tokens, int E, int K,
     if (t >= n_tokens) return;
     const T* row = logits + (size_t)t * E;
 
+    typedef typename SelKey<T>::type key_t;
     float v[VPT];
-    unsigned long long key[VPT];
+    key_t key[VPT];
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
         int e = lane + 64 * j;
         bool ok = e < E;
         v[j] = ok ? ElemTraits<T>::load1(row + (ok ? e : 0)) : -INFINITY;
-        key[j] = ok ? sel_key(v[j], e) : 0ull;
+        key[j] = ok ? SelKey<T>::make(v[j], e) : (key_t)0;
     }
 
     // K rounds of wave-wide arg-max; a taken entry's key drops to 0
@@ -70,16 +116,16 @@ router_topk_fwd_kernel(const T* __restrict__ logits, int n_tokens, int E, int K,
     int top_e = 0;       // lane k keeps the k-th selected expert
     float row_max = 0.f;
     for (int k = 0; k < K; ++k) {
-        unsigned long long best = key[0];
+        key_t best = key[0];
 #pragma unroll
         for (int j = 1; j < VPT; ++j) best = key[j] > best ? key[j] : best;
-        best = wave_max_u64(best);
-        int e_sel = (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull));
+        best = wave_max_key(best);
+        int e_sel = SelKey<T>::index(best);
         float v_sel = 0.f;
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
             if (lane + 64 * j == e_sel) {
-                key[j] = 0ull;
+                key[j] = (key_t)0;
                 v_sel = v[j];
             }
         }
@@ -107,6 +153,7 @@ router_topk_fwd_kernel(const T* __restrict__ logits, int n_tokens, int E, int K,
         int e = lane + 64 * j;
         if (e < E) prow[e] = ex[j] / z;
     }
+    // (the division stays an IEEE division: the probabilities are compared with the library softmax)
 
     float p_sel = (lane < K) ? expf(top_v - row_max) / z : 0.f;
     float s = p_sel;

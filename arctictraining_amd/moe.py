@@ -184,7 +184,13 @@ class _ExpertLayerFn(torch.autograd.Function):
                 bad = ((assign < 0) | (assign >= E)).any()
                 if bool(bad):
                     raise RuntimeError(f"routing_replay_assignments holds expert ids outside [0, {E})")
-        counts, offsets, token_of, slot_of, row_of, scores_perm = ops.permute_plan(assign, E, scores)
+        # the four row-grouped GEMMs of a step share one tile map: the permutation plan builds it
+        # (its scan kernel holds the offsets), the workspace is kept for backward
+        cfg = opts["tile_cfg"]
+        ws = ops.gemm_workspace(T * K, E, x.device)
+        counts, offsets, token_of, slot_of, row_of, scores_perm = ops.permute_plan(
+            assign, E, scores, gemm_workspace=ws, gemm_dtype=x.dtype, tile_cfg=cfg
+        )
         timers.stop("router")
 
         # The gather x[token_of] (moe.py:356) happens inside the GEMMs' A loads: the routed copy
@@ -192,12 +198,9 @@ class _ExpertLayerFn(torch.autograd.Function):
         # the gate_up GEMM) instead of its output: the down projection is linear, so
         # (s * inter) @ W_down == s * (inter @ W_down), and the combine becomes a plain sum.
         timers.start("groupGeMM")
-        cfg = opts["tile_cfg"]
-        # the four row-grouped GEMMs of a step share one tile map: built once here, kept for backward
-        ws = ops.gemm_workspace(T * K, E, x.device)
         gate_up, inter_s = ops.grouped_gemm_gateup_act_fwd(
             x, w_gate_up, offsets, opts["act"], a_row_map=token_of, n_rows=T * K, tile_cfg=cfg, row_scale=scores_perm,
-            workspace=ws,
+            workspace=ws, map_ready=True,
         )
         out_s = ops.grouped_gemm_nn(inter_s, w_down, offsets, tile_cfg=cfg, workspace=ws, map_ready=True)
         timers.stop("groupGeMM")

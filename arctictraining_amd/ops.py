@@ -76,9 +76,12 @@ def router_bwd(d_scores, probs, topk_idx, counts, out_dtype, normalize: bool, lb
     return d_logits
 
 
-def permute_plan(assign: torch.Tensor, num_experts: int, scores: Optional[torch.Tensor] = None):
+def permute_plan(assign: torch.Tensor, num_experts: int, scores: Optional[torch.Tensor] = None,
+                 gemm_workspace: Optional[torch.Tensor] = None, gemm_dtype: Optional[torch.dtype] = None, tile_cfg: int = 0):
     """assign [T,K] i32 -> counts [E], offsets [E+1], token_of [R], slot_of [R], row_of [T,K] (all i32) and,
-    when scores [T,K] f32 is given, scores_perm [R] f32 (else None)."""
+    when scores [T,K] f32 is given, scores_perm [R] f32 (else None).  With gemm_workspace (and the
+    dtype / tile_cfg of the row-grouped GEMMs that will use it) the plan also builds their tile map
+    there, so that each of them can be called with map_ready=True."""
     lib = _lib.load()
     _chk(assign, "assign", torch.int32)
     T, K = assign.shape
@@ -94,6 +97,15 @@ def permute_plan(assign: torch.Tensor, num_experts: int, scores: Optional[torch.
         scores_perm = torch.empty(R, dtype=torch.float32, device=dev)
     ws_bytes = lib.amoe_permute_workspace_bytes(R, E)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    if gemm_workspace is not None:
+        _chk(gemm_workspace, "gemm_workspace", torch.uint8)
+        rc = lib.amoe_permute_plan_tiled(
+            assign.data_ptr(), _ptr(scores), T, K, E, counts.data_ptr(), offsets.data_ptr(), token_of.data_ptr(),
+            slot_of.data_ptr(), row_of.data_ptr(), _ptr(scores_perm), ws.data_ptr(), ws.numel(), gemm_workspace.data_ptr(),
+            gemm_workspace.numel(), F32 if gemm_dtype == torch.float32 else BF16, tile_cfg, _stream()
+        )
+        _lib.check(rc, "amoe_permute_plan_tiled")
+        return counts, offsets, token_of, slot_of, row_of, scores_perm
     rc = lib.amoe_permute_plan(
         assign.data_ptr(), _ptr(scores), T, K, E, counts.data_ptr(), offsets.data_ptr(), token_of.data_ptr(),
         slot_of.data_ptr(), row_of.data_ptr(), _ptr(scores_perm), ws.data_ptr(), ws.numel(), _stream()

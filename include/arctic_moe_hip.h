@@ -90,6 +90,18 @@ int amoe_permute_plan(const int32_t* assign, const float* scores, int T, int K, 
                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * amoe_permute_plan that also builds the tile map of the row-grouped GEMMs which will run over
+ * its offsets (its scan kernel holds the offsets anyway, so the map costs no launch of its own).
+ * gemm_workspace is the workspace those GEMMs will be given (amoe_grouped_gemm_workspace_bytes
+ * (T*K, E) bytes); dtype and tile_cfg are theirs.  Every row-grouped GEMM over these offsets may
+ * then pass tile_cfg | AMOE_TILE_MAP_READY.
+ */
+int amoe_permute_plan_tiled(const int32_t* assign, const float* scores, int T, int K, int E, int32_t* counts,
+                            int32_t* offsets, int32_t* token_of, int32_t* slot_of, int32_t* row_of, float* scores_perm,
+                            void* workspace, size_t workspace_bytes, void* gemm_workspace, size_t gemm_workspace_bytes,
+                            int dtype, int tile_cfg, void* stream);
+
+/*
  * amoe_permute_plan for callers that cannot allocate device memory (code recorded into a HIP
  * graph, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  Same arguments and results as amoe_permute_plan without the workspace: the

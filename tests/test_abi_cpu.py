@@ -74,6 +74,16 @@ def test_permute_argument_errors(lib):
     assert lib.amoe_permute_plan(P, None, 4, 2, 600, P, P, P, P, P, None, P, 1 << 20, None) == -2
 
 
+def test_permute_tiled_argument_errors(lib):
+    f = lib.amoe_permute_plan_tiled
+    big = 1 << 20
+    assert f(P, None, 4, 2, 8, P, P, P, P, P, None, P, big, None, big, 1, 0, None) == -1   # no GEMM workspace
+    assert f(P, None, 4, 2, 8, P, P, P, P, P, None, P, big, P, 8, 1, 0, None) == -3        # GEMM workspace too small
+    assert f(P, None, 4, 2, 8, P, P, P, P, P, None, P, big, P, big, 5, 0, None) == -1      # dtype
+    assert f(P, None, 4, 2, 8, P, P, P, P, P, None, P, big, P, big, 1, 4, None) == -1      # tile_cfg
+    assert f(P, None, 4, 2, 8, P, P, P, P, P, None, P, 0, P, big, 1, 0, None) == -3        # plan workspace too small
+
+
 def test_permute_static_argument_errors(lib):
     assert lib.amoe_permute_plan_static(None, None, 4, 2, 8, P, P, P, P, P, None, None) == -1
     assert lib.amoe_permute_plan_static(P, None, 4, 2, 8, P, P, P, P, P, P, None) == -1  # scores_perm without scores

@@ -475,3 +475,33 @@ def test_grouped_gemm_shared_tile_map(ops, gpu_device, dtype):
     assert torch.equal(d_again, ops.grouped_gemm_nt(A2, B, offs))
     with pytest.raises(RuntimeError, match="workspace"):
         ops.grouped_gemm_nn(A, B, offs, map_ready=True)
+
+
+@pytest.mark.parametrize("dtype,cfg", [(torch.bfloat16, 0), (torch.bfloat16, 1), (torch.float32, 0)])
+def test_permute_plan_builds_the_gemm_tile_map(ops, gpu_device, dtype, cfg):
+    """The plan can build the row-grouped GEMMs' tile map as a by-product of its scan kernel: a GEMM
+    that reuses it (map_ready) gives exactly the result of one that builds its own, with empty
+    experts, one-row experts and experts of several tiles; the plan's own outputs are unchanged."""
+    g = torch.Generator().manual_seed(31)
+    T, K, E, Kd, N = 1700, 3, 9, 96, 160
+    assign = torch.randint(0, E, (T, K), generator=g)
+    assign[assign == 4] = 5            # expert 4 empty
+    assign[assign == 7] = 0
+    assign[0, 0] = 7                   # expert 7 holds one row
+    a32 = assign.to(torch.int32).to(gpu_device)
+    R = T * K
+    ws = ops.gemm_workspace(R, E, gpu_device)
+    ws.fill_(0xAB)                     # stale bytes must not survive
+    plain = ops.permute_plan(a32, E)
+    tiled = ops.permute_plan(a32, E, gemm_workspace=ws, gemm_dtype=dtype, tile_cfg=cfg)
+    for a, b in zip(plain[:5], tiled[:5]):
+        assert torch.equal(a, b)
+    offs = tiled[1]
+    assert int(tiled[0][4]) == 0 and int(tiled[0][7]) == 1
+    A = torch.randn(R, Kd, generator=g).to(dtype).to(gpu_device)
+    B = (torch.randn(E, Kd, N, generator=g) * 0.1).to(dtype).to(gpu_device)
+    assert torch.equal(ops.grouped_gemm_nn(A, B, offs, tile_cfg=cfg, workspace=ws, map_ready=True),
+                       ops.grouped_gemm_nn(A, B, offs, tile_cfg=cfg))
+    A2 = torch.randn(R, N, generator=g).to(dtype).to(gpu_device)
+    assert torch.equal(ops.grouped_gemm_nt(A2, B, offs, tile_cfg=cfg, workspace=ws, map_ready=True),
+                       ops.grouped_gemm_nt(A2, B, offs, tile_cfg=cfg))
