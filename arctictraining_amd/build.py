@@ -65,6 +65,24 @@ def _check_gemm_assembly() -> None:
     asm_check.check_assembly(asm, min_kernels=20)
 
 
+STAMP_PATH = os.path.join(LIB_DIR, "build_commit.txt")
+
+
+def _stamp_commit() -> None:
+    """Record which commit the library was built from next to it (the stamp travels with the built
+    library to machines that have no git history; measurements quote it)."""
+    try:
+        root = os.path.dirname(PKG_DIR)
+        head = subprocess.run(["git", "-C", root, "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True, timeout=10)
+        dirty = subprocess.run(["git", "-C", root, "status", "--porcelain", "--untracked-files=no"], capture_output=True,
+                               text=True, timeout=10)
+        if head.returncode == 0 and head.stdout.strip():
+            with open(STAMP_PATH, "w") as fh:
+                fh.write(head.stdout.strip() + ("+uncommitted" if dirty.stdout.strip() else "") + "\n")
+    except Exception:
+        pass  # no git here: leave whatever stamp came with the tree
+
+
 def build(force: bool = True, jobs: int = 6) -> str:
     """Compile every HIP source, check the GEMM assembly, and link the shared library; returns its path."""
     os.makedirs(OBJ_DIR, exist_ok=True)
@@ -86,6 +104,7 @@ def build(force: bool = True, jobs: int = 6) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
+    _stamp_commit()
     return LIB_PATH
 
 

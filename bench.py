@@ -85,10 +85,19 @@ def time_op(fn, iters, torch):
 
 
 def git_head():
+    """The commit of the running tree: from git when the history is here, otherwise the stamp that
+    the library build left beside the library it built."""
     try:
-        return subprocess.run(["git", "-C", ROOT, "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True,
-                              timeout=10).stdout.strip() or None
+        out = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True,
+                             timeout=10).stdout.strip()
+        if out:
+            return out
     except Exception:
+        pass
+    try:
+        with open(os.path.join(ROOT, "arctictraining_amd", "lib", "build_commit.txt")) as fh:
+            return fh.read().strip() or None
+    except OSError:
         return None
 
 
