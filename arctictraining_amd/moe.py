@@ -160,6 +160,35 @@ def _router_weight_grad(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor
     return _dense_weight_grad(d_logits, x, tile_cfg=1, tile=128)  # 128x128 tiles
 
 
+def _route(x, router_gate, replay, opts):
+    """Router linear map, softmax / top-k, and the permutation plan with the tile map of the
+    row-grouped GEMMs (moe.py:231-233, 359-382).  Returns logits, probs, topk_idx, scores [T,K],
+    the GEMM workspace that holds the tile map, and the plan (counts, offsets, token_of, slot_of,
+    row_of, scores_perm)."""
+    T = x.shape[0]
+    E, K = opts["num_experts"], opts["top_k"]
+    timers: PhaseTimers = opts["timers"]
+    timers.start("router")
+    logits = torch.matmul(x, router_gate.t())  # plain library GEMM, moe.py:233
+    probs, topk_idx, scores = ops.router_topk_fwd(logits, K, opts["normalize"])
+    assign = topk_idx
+    if replay is not None:
+        assign = replay.to(torch.int32).contiguous()
+        if os.environ.get("AMOE_CHECK_REPLAY") == "1":
+            # The reference's one_hot(..., num_classes=E) raises on an expert id outside [0, E)
+            # (moe.py:374); the permutation kernels clamp such ids for memory safety instead.  This
+            # opt-in check restores the error at the price of a host synchronisation.
+            bad = ((assign < 0) | (assign >= E)).any()
+            if bool(bad):
+                raise RuntimeError(f"routing_replay_assignments holds expert ids outside [0, {E})")
+    # the row-grouped GEMMs of a step share one tile map: the permutation plan builds it (its
+    # scan kernel holds the offsets), the workspace is kept for backward
+    ws = ops.gemm_workspace(T * K, E, x.device)
+    plan = ops.permute_plan(assign, E, scores, gemm_workspace=ws, gemm_dtype=x.dtype, tile_cfg=opts["tile_cfg"])
+    timers.stop("router")
+    return logits, probs, topk_idx, scores, ws, plan
+
+
 class _ExpertLayerFn(torch.autograd.Function):
     """router top-k -> permutation -> grouped gated FFN -> weighted combine, and the
     gradients of all of it (the autograd of moe.py:231-233, 340-411, 176-193, 450-461 plus
@@ -170,28 +199,10 @@ class _ExpertLayerFn(torch.autograd.Function):
         T, H = x.shape
         E, K = opts["num_experts"], opts["top_k"]
         timers: PhaseTimers = opts["timers"]
-
-        timers.start("router")
-        logits = torch.matmul(x, router_gate.t())  # plain library GEMM, moe.py:233
-        probs, topk_idx, scores = ops.router_topk_fwd(logits, K, opts["normalize"])
-        assign = topk_idx
-        if replay is not None:
-            assign = replay.to(torch.int32).contiguous()
-            if os.environ.get("AMOE_CHECK_REPLAY") == "1":
-                # The reference's one_hot(..., num_classes=E) raises on an expert id outside [0, E)
-                # (moe.py:374); the permutation kernels clamp such ids for memory safety instead.  This
-                # opt-in check restores the error at the price of a host synchronisation.
-                bad = ((assign < 0) | (assign >= E)).any()
-                if bool(bad):
-                    raise RuntimeError(f"routing_replay_assignments holds expert ids outside [0, {E})")
-        # the four row-grouped GEMMs of a step share one tile map: the permutation plan builds it
-        # (its scan kernel holds the offsets), the workspace is kept for backward
         cfg = opts["tile_cfg"]
-        ws = ops.gemm_workspace(T * K, E, x.device)
-        counts, offsets, token_of, slot_of, row_of, scores_perm = ops.permute_plan(
-            assign, E, scores, gemm_workspace=ws, gemm_dtype=x.dtype, tile_cfg=cfg
+        logits, probs, topk_idx, scores, ws, (counts, offsets, token_of, slot_of, row_of, scores_perm) = _route(
+            x, router_gate, replay, opts
         )
-        timers.stop("router")
 
         # The gather x[token_of] (moe.py:356) happens inside the GEMMs' A loads: the routed copy
         # of the activations is never written.  The score of a routed row multiplies the expert's intermediate activation (epilogue of
@@ -327,6 +338,115 @@ class _ExpertLayerFn(torch.autograd.Function):
         return dx, d_router_gate, d_w_gate_up, d_w_down, d_sh_gate_up, d_sh_down, d_sh_out_gate, None, None
 
 
+class _UngatedExpertLayerFn(torch.autograd.Function):
+    """The layer with is_gated=False (moe.py:101-106, 188-191, 306-311): an expert is two plain
+    linear maps, out = (x @ W_up[e]) @ W_down[e] with W_up [E,H,I] -- the reference applies its
+    activation only inside the gated branch -- and the routing scores weight the combine
+    (moe.py:450-461).  Same routing, permutation, load-balance hook and gradients as the gated
+    layer; the grouped GEMMs run without an activation epilogue."""
+
+    @staticmethod
+    def forward(ctx, x, router_gate, w_up, w_down, sh_up, sh_down, sh_out_gate, replay, opts):
+        T, H = x.shape
+        K = opts["top_k"]
+        timers: PhaseTimers = opts["timers"]
+        cfg = opts["tile_cfg"]
+        logits, probs, topk_idx, scores, ws, (counts, offsets, token_of, slot_of, row_of, scores_perm) = _route(
+            x, router_gate, replay, opts
+        )
+        timers.start("groupGeMM")
+        inter = ops.grouped_gemm_nn(x, w_up, offsets, a_row_map=token_of, n_rows=T * K, tile_cfg=cfg, workspace=ws,
+                                    map_ready=True)
+        out = ops.grouped_gemm_nn(inter, w_down, offsets, tile_cfg=cfg, workspace=ws, map_ready=True)
+        timers.stop("groupGeMM")
+        timers.start("moe-combine")
+        y = ops.combine_fwd(out, row_of, scores)
+        timers.stop("moe-combine")
+
+        shared = sh_up is not None
+        sh_inter = sh_out = sh_sig = None
+        if shared:
+            # dense linear maps over all T tokens: plain library GEMMs, like the reference's
+            timers.start("shared-expert")
+            sh_inter = torch.matmul(x, sh_up)
+            sh_out = torch.matmul(sh_inter, sh_down)
+            sh_sig = torch.sigmoid(torch.matmul(x, sh_out_gate))  # [T,1]
+            y = y + sh_out * sh_sig
+            timers.stop("shared-expert")
+
+        ctx.opts = opts
+        ctx.shared = shared
+        ctx.gemm_ws = ws
+        ctx.save_for_backward(x, router_gate, w_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, scores,
+                              inter, out, sh_up, sh_down, sh_out_gate, sh_inter, sh_out, sh_sig)
+        if opts["want_scores"]:
+            scores_out = scores_perm.to(x.dtype)
+        else:
+            scores_out = scores_perm.new_empty(0)
+            ctx.mark_non_differentiable(scores_out)
+        ctx.set_materialize_grads(False)
+        cap = opts.get("capture")
+        if cap is not None:
+            cap.update(logits=logits, probs=probs, topk_idx=topk_idx, scores=scores, counts=counts, offsets=offsets,
+                       token_of=token_of, slot_of=slot_of, row_of=row_of)
+        return y, scores_out
+
+    @staticmethod
+    def backward(ctx, dy, ds_perm):
+        (x, router_gate, w_up, w_down, probs, topk_idx, counts, offsets, row_of, token_of, scores,
+         inter, out, sh_up, sh_down, sh_out_gate, sh_inter, sh_out, sh_sig) = ctx.saved_tensors
+        opts = ctx.opts
+        E, K = opts["num_experts"], opts["top_k"]
+        T = x.shape[0]
+        cfg = opts["tile_cfg"]
+        if dy is None and ds_perm is None:
+            return (None,) * 9
+        dy = torch.zeros_like(x) if dy is None else dy.contiguous()
+        ws = ctx.gemm_ws  # still holds the forward's tile map
+
+        # d_out[r] = s_r * dy[token_of[r]],  d_scores[t,k] = <dy[t], out[row_of[t,k]]>
+        d_out, d_scores = ops.combine_bwd(dy, out, row_of, scores)
+        if ds_perm is not None:
+            d_scores = d_scores + ds_perm.float()[row_of.long()]
+        d_inter = ops.grouped_gemm_nt(d_out, w_down, offsets, tile_cfg=cfg, workspace=ws, map_ready=True)
+        d_w_down = ops.grouped_gemm_wgrad(inter, d_out, offsets, E, tile_cfg=cfg) if ctx.needs_input_grad[3] else None
+        d_w_up = None
+        if ctx.needs_input_grad[2]:
+            d_w_up = ops.grouped_gemm_wgrad(x, d_inter, offsets, E, tile_cfg=cfg, a_row_map=token_of)
+
+        d_logits = ops.router_bwd(
+            d_scores, probs, topk_idx, counts, x.dtype, opts["normalize"], opts["loss_coeff"] / T / opts["ep_size"]
+        )
+        d_router_gate = _router_weight_grad(d_logits, x) if ctx.needs_input_grad[1] else None
+        cap = opts.get("capture")
+        if cap is not None:
+            cap.update(d_scores=d_scores, d_logits=d_logits)
+
+        d_sh_up = d_sh_down = d_sh_out_gate = d_sh_inter = d_pre = None
+        if ctx.shared:
+            d_sh_out = dy * sh_sig
+            d_sig = (dy.float() * sh_out.float()).sum(dim=1, keepdim=True)
+            sig = sh_sig.float()
+            d_pre = (d_sig * sig * (1.0 - sig)).to(x.dtype)  # [T,1]
+            d_sh_inter = torch.matmul(d_sh_out, sh_down.t())
+            if ctx.needs_input_grad[5]:
+                d_sh_down = torch.matmul(sh_inter.t(), d_sh_out)
+            if ctx.needs_input_grad[4]:
+                d_sh_up = torch.matmul(x.t(), d_sh_inter)
+            if ctx.needs_input_grad[6]:
+                d_sh_out_gate = torch.matmul(x.t(), d_pre)
+
+        dx = None
+        if ctx.needs_input_grad[0]:
+            d_xp = ops.grouped_gemm_nt(d_inter, w_up, offsets, tile_cfg=cfg, workspace=ws, map_ready=True)
+            dx_dense = torch.matmul(d_logits, router_gate)
+            if ctx.shared:
+                dx_dense.addmm_(d_pre, sh_out_gate.t())
+                dx_dense.addmm_(d_sh_inter, sh_up.t())
+            dx = ops.gather_rows_bwd(d_xp, row_of, addend=dx_dense)
+        return dx, d_router_gate, d_w_up, d_w_down, d_sh_up, d_sh_down, d_sh_out_gate, None, None
+
+
 class ArcticMoE(nn.Module):
     """Mixture-of-experts layer with the reference's surface (moe.py:63-323).
 
@@ -350,8 +470,7 @@ class ArcticMoE(nn.Module):
         self.use_custom_kernel = getattr(config, "use_custom_moe_kernel", False)
         if self.ep_size != 1:
             raise NotImplementedError("this build runs the expert layer on one GPU (ep_size must be 1)")
-        if not getattr(config, "is_gated", True):
-            raise NotImplementedError("only gated expert FFNs are supported (is_gated=True)")
+        self.is_gated = bool(getattr(config, "is_gated", True))
         self._act_code = classify_activation(config.act_fn)
 
         self.timers = PhaseTimers()
@@ -362,15 +481,17 @@ class ArcticMoE(nn.Module):
         self.capture = None  # set to a dict to receive the routing intermediates of each forward
 
         dt = self.input_dtype
+        # gate and up projection interleaved when gated, one plain projection otherwise (moe.py:101-106)
+        up_cols = (2 if self.is_gated else 1) * self.intermediate_dim
         self.router_gate = nn.Parameter(torch.empty((self.num_experts, self.model_dim), dtype=dt))
         self.expert_gate_up = nn.Parameter(
-            torch.empty((self.num_local_experts, self.model_dim, 2 * self.intermediate_dim), dtype=dt)
+            torch.empty((self.num_local_experts, self.model_dim, up_cols), dtype=dt)
         )
         self.gate_scale = 1.0
         self.up_scale = 0.0
         self.expert_down = nn.Parameter(torch.empty((self.num_local_experts, self.intermediate_dim, self.model_dim), dtype=dt))
         if getattr(config, "use_shared_expert", False):
-            self.shared_expert_gate_up = nn.Parameter(torch.empty((self.model_dim, 2 * self.intermediate_dim), dtype=dt))
+            self.shared_expert_gate_up = nn.Parameter(torch.empty((self.model_dim, up_cols), dtype=dt))
             self.shared_expert_down = nn.Parameter(torch.empty((self.intermediate_dim, self.model_dim), dtype=dt))
             self.shared_expert_output_gate = nn.Parameter(torch.empty(self.model_dim, 1, dtype=dt))
         self.enable_routing_replay = getattr(config, "enable_routing_replay", False)
@@ -426,7 +547,8 @@ class ArcticMoE(nn.Module):
             shared = (self.shared_expert_gate_up, self.shared_expert_down, self.shared_expert_output_gate)
         # the kernels are launched on the current device's current stream: make x's device current
         with torch.cuda.device(x.device) if x.is_cuda else contextlib.nullcontext():
-            output, scores = _ExpertLayerFn.apply(
+            layer_fn = _ExpertLayerFn if self.is_gated else _UngatedExpertLayerFn
+            output, scores = layer_fn.apply(
                 x, self.router_gate, self.expert_gate_up, self.expert_down, *shared, replay, opts
             )
         output = output.reshape(orig_shape)

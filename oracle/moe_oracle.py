@@ -20,6 +20,7 @@ reference tree):
   row gather           arctic_training/model/moe/moe.py:353-357
   grouped GEMM         arctic_training/model/moe/moe.py:54-60
   gated expert FFN     arctic_training/model/moe/moe.py:176-193 (scale constants :110-111)
+  expert FFN, no gate  arctic_training/model/moe/moe.py:101-106, 188-191 (is_gated=False: no activation)
   weighted combine     arctic_training/model/moe/moe.py:450-461
   shared expert        arctic_training/model/moe/moe.py:305-314 (parameters :116-130)
   weight layout        arctic_training/model/moe/utils.py:249-266
@@ -37,7 +38,9 @@ installed third-party HF block instead):
                         the invariants and a worked example
   grouped_gemm          per-expert fp64 matmul on the same row ranges; empty
                         groups leave zero rows
-  expert_ffn            de-interleaved chunk formulation; silu closed form
+  expert_ffn            de-interleaved chunk formulation; silu closed form;
+                        is_gated=False: token-major dense closed form of the
+                        whole layer (two products, no activation)
   combine               dense token-major sum
   shared_expert         the installed transformers Qwen2MoeSparseMoeBlock
                         (shared MLP + sigmoid gate) after weight-layout mapping,
@@ -70,6 +73,7 @@ class OracleConfig:
     loss_coeff: float = 0.01
     ep_size: int = 1
     act: str = "silu"
+    is_gated: bool = True
 
 
 def activation(name: str) -> Callable[[torch.Tensor], torch.Tensor]:
@@ -226,12 +230,17 @@ def grouped_gemm(A: torch.Tensor, B: torch.Tensor, rows_cumsum: torch.Tensor) ->
     return out
 
 
-def expert_ffn(xp: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, rows_cumsum, act: str):
+def expert_ffn(xp: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, rows_cumsum, act: str,
+               is_gated: bool = True):
     """moe.py:176-193 -- gate in the even, up in the odd columns of the first
     GEMM's output; inter = (up + 0.0) * act(gate * 1.0); second GEMM.
-    Returns (gate_up, inter, out)."""
+    Returns (gate_up, inter, out).  With is_gated=False (w_gate_up [E,H,I], moe.py:101-106) the
+    first GEMM's output goes to the second as it is: the activation sits inside the gated branch
+    only (moe.py:188-191)."""
     fn = activation(act)
     gu = grouped_gemm(xp, w_gate_up, rows_cumsum)
+    if not is_gated:
+        return gu, gu, grouped_gemm(gu, w_down, rows_cumsum)
     g, u = gu[..., 0::2], gu[..., 1::2]
     inter = (u + 0.0) * fn(g * 1.0)
     out = grouped_gemm(inter, w_down, rows_cumsum)
@@ -245,14 +254,16 @@ def combine(moe_out: torch.Tensor, token_ids: torch.Tensor, scores_perm: torch.T
     return y.index_add(0, token_ids, moe_out * scores_perm[:, None])
 
 
-def shared_expert(x2d: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, w_out_gate: torch.Tensor, act: str):
+def shared_expert(x2d: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, w_out_gate: torch.Tensor, act: str,
+                  is_gated: bool = True):
     """moe.py:305-314 -- a dense gated FFN every token goes through, scaled per token by a
     sigmoid gate: (up * act(gate)) @ W_down * sigmoid(x @ w_out_gate).  w_gate_up [H, 2I] has the
     gate in the even and the up projection in the odd columns, w_down is [I, H], w_out_gate [H, 1]."""
     fn = activation(act)
     s_inter = torch.matmul(x2d, w_gate_up)
-    s_gate, s_up = s_inter[..., 0::2], s_inter[..., 1::2]
-    s_inter = s_up * fn(s_gate)
+    if is_gated:  # moe.py:308-310; without the gate the first product feeds the second unchanged
+        s_gate, s_up = s_inter[..., 0::2], s_inter[..., 1::2]
+        s_inter = s_up * fn(s_gate)
     s_out = torch.matmul(s_inter, w_down)
     s_out_gate = torch.matmul(x2d, w_out_gate)
     return s_out * torch.sigmoid(s_out_gate)
@@ -321,10 +332,10 @@ def forward(
 
     xp = x2d[g["token_ids"]]
     cumsum = g["counts"].cumsum(0)
-    gu, inter, out = expert_ffn(xp, expert_gate_up, expert_down, cumsum, cfg.act)
+    gu, inter, out = expert_ffn(xp, expert_gate_up, expert_down, cumsum, cfg.act, cfg.is_gated)
     y = combine(out, g["token_ids"], g["scores_perm"], cfg.top_k)
     if shared is not None:
-        y = y + shared_expert(x2d, *shared, cfg.act)
+        y = y + shared_expert(x2d, *shared, cfg.act, cfg.is_gated)
     res = dict(g)
     res.update(logits=logits, xp=xp, gate_up=gu, inter=inter, moe_out=out, y=y.reshape(orig_shape), cumsum=cumsum)
     return res
@@ -385,7 +396,7 @@ def analytic_backward(res: Dict[str, torch.Tensor], x2d, router_gate, expert_gat
     `forward` in an exact mode (float32/float64); the formulas are the
     derivatives of moe.py:233, :361-366, :356, :187-192, :460 and the hook at
     :393-406.  SiLU only."""
-    assert cfg.act == "silu"
+    assert cfg.act == "silu" and cfg.is_gated
     dt = res["y"].dtype
     x2d, router_gate, expert_gate_up, expert_down, dy2d = (
         t.detach().to(dt) for t in (x2d, router_gate, expert_gate_up, expert_down, dy2d)

@@ -208,6 +208,67 @@ def test_layer_shared_expert(gpu_device, dtype, T, H, E, K, I, act):
     assert O.rel_l2(got["y"], routed_only["y"]) > 10 * tol
 
 
+@pytest.mark.parametrize(
+    "dtype,T,H,E,K,I,shared",
+    [
+        (torch.float32, 200, 64, 4, 2, 96, False),
+        (torch.bfloat16, 1500, 256, 16, 4, 384, False),
+        (torch.bfloat16, 1024, 256, 8, 2, 128, True),
+        (torch.float32, 128, 64, 4, 2, 32, True),
+    ],
+    ids=["fp32", "bf16", "bf16_shared", "fp32_shared"],
+)
+def test_layer_without_gate(gpu_device, dtype, T, H, E, K, I, shared):
+    """is_gated=False (moe.py:101-106, 188-191, 306-311): expert_gate_up is [E,H,I] and an expert is
+    (x @ W_up) @ W_down with nothing in between; the routing scores weight the combine.  Output,
+    returned scores and every gradient (with a gradient flowing into the returned scores) against
+    the oracle."""
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=21)
+    wup = wgu[:, :, :I].contiguous()   # a plain [E,H,I] projection
+    layer = build_layer(dtype, H, E, K, I, gpu_device, is_gated=False, use_shared_expert=shared,
+                        return_router_scores=True)
+    assert tuple(layer.expert_gate_up.shape) == (E, H, I)
+    sh = None
+    if shared:
+        assert tuple(layer.shared_expert_gate_up.shape) == (H, I)
+        g = torch.Generator().manual_seed(22)
+        sh = tuple((torch.randn(s, generator=g) * 0.05).to(dtype) for s in ((H, I), (I, H), (H, 1)))
+        with torch.no_grad():
+            layer.shared_expert_gate_up.copy_(sh[0])
+            layer.shared_expert_down.copy_(sh[1])
+            layer.shared_expert_output_gate.copy_(sh[2])
+    with torch.no_grad():
+        layer.router_gate.copy_(wr)
+        layer.expert_gate_up.copy_(wup)
+        layer.expert_down.copy_(wd)
+    layer.capture = {}
+    g = torch.Generator().manual_seed(23)
+    d_sp = torch.randn(T * K, generator=g)
+    xg = x.to(gpu_device).requires_grad_(True)
+    y, sp = layer(xg)
+    torch.autograd.backward([y, sp], [dy.to(gpu_device), d_sp.to(dtype).to(gpu_device)])
+    torch.cuda.synchronize()
+    cap = {k: v.cpu() for k, v in layer.capture.items()}
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001, is_gated=False)
+    ref = O.forward_backward(
+        x, wr, wup, wd, dy, ocfg, compute_dtype=torch.float64, logits_for_selection=cap["logits"], shared=sh,
+        d_scores_perm=d_sp.to(dtype),
+    )
+    assert torch.equal(cap["topk_idx"].long(), ref["topk_idx"])
+    assert torch.equal(cap["slot_of"].long(), ref["perm"])
+    got = dict(y=y.detach().cpu(), dx=xg.grad.cpu(), d_router_gate=layer.router_gate.grad.cpu(),
+               d_expert_gate_up=layer.expert_gate_up.grad.cpu(), d_expert_down=layer.expert_down.grad.cpu())
+    errs = {k: O.rel_l2(v, ref[k]) for k, v in got.items()}
+    print("rel-L2:", {k: f"{v:.2e}" for k, v in errs.items()}, flush=True)
+    for k, v in errs.items():
+        assert v <= tol, f"{k}: rel-L2 {v:.3e} > {tol}"
+    assert O.rel_l2(sp.detach().float().cpu(), ref["scores_perm"]) <= tol
+    if shared:
+        for name in ("shared_expert_gate_up", "shared_expert_down", "shared_expert_output_gate"):
+            assert O.rel_l2(getattr(layer, name).grad.cpu(), ref["d_" + name]) <= tol, name
+
+
 def test_layer_is_deterministic(gpu_device):
     dtype, T, H, E, K, I = torch.bfloat16, 1024, 256, 32, 4, 128
     x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=13)

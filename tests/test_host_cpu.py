@@ -29,3 +29,20 @@ def test_activation_classification():
     assert moe.classify_activation(F.gelu) == ops.ACT_GELU
     assert moe.classify_activation(F.relu) == ops.ACT_RELU
     assert moe.classify_activation(lambda x: x * torch.sigmoid(1.702 * x)) == ops.ACT_GPT_OSS
+
+
+def test_layer_without_gate_parameter_shapes():
+    """is_gated=False: one plain [E,H,I] projection instead of the interleaved [E,H,2I] pair
+    (moe.py:101-106), the shared expert likewise (:118-124)."""
+    import torch.nn.functional as F
+
+    from arctictraining_amd import ArcticMoE, MoEConfig
+
+    cfg = MoEConfig(act_fn=F.silu, input_dtype=torch.float32, intermediate_dim=6, model_dim=8, normalize_topk_scores=True,
+                    num_experts=4, top_k=2, is_gated=False, use_shared_expert=True)
+    m = ArcticMoE(cfg)
+    assert tuple(m.expert_gate_up.shape) == (4, 8, 6) and tuple(m.expert_down.shape) == (4, 6, 8)
+    assert tuple(m.shared_expert_gate_up.shape) == (8, 6)
+    gated = ArcticMoE(MoEConfig(act_fn=F.silu, input_dtype=torch.float32, intermediate_dim=6, model_dim=8,
+                                normalize_topk_scores=True, num_experts=4, top_k=2))
+    assert tuple(gated.expert_gate_up.shape) == (4, 8, 12)

@@ -323,6 +323,39 @@ def test_shared_expert_closed_form():
     assert abs(float(swapped) - want) > 1e-3
 
 
+def test_layer_without_gate_closed_form():
+    """is_gated=False (moe.py:101-106, 188-191, 306-311): the layer is linear in x between the
+    router and the combine.  Checked against a token-major dense evaluation that shares only the
+    routing decision (indices and scores) with the oracle:
+    y[t] = sum_k s[t,k] * (x[t] @ W_up[e] @ W_down[e]) + (x[t] @ S_up @ S_down) * sigmoid(x[t] @ s_o).
+    A stray activation, a de-interleave of the [E,H,I] projection or a missing score would fail it."""
+    T, H, E, K, I = 23, 12, 5, 2, 7
+    g = torch.Generator().manual_seed(5)
+    x, wr = torch.randn(T, H, generator=g, dtype=torch.float64), torch.randn(E, H, generator=g, dtype=torch.float64)
+    wup = torch.randn(E, H, I, generator=g, dtype=torch.float64)
+    wd = torch.randn(E, I, H, generator=g, dtype=torch.float64)
+    sh = (torch.randn(H, I, generator=g, dtype=torch.float64), torch.randn(I, H, generator=g, dtype=torch.float64),
+          torch.randn(H, 1, generator=g, dtype=torch.float64))
+    cfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, is_gated=False)
+    for shared in (None, sh):
+        res = O.forward(x, wr, wup, wd, cfg, shared=shared)
+        probs = torch.softmax(x @ wr.t(), dim=-1)
+        s, idx = probs.topk(K, dim=-1)
+        s = s / s.sum(-1, keepdim=True)
+        want = torch.zeros(T, H, dtype=torch.float64)
+        for t in range(T):
+            for k in range(K):
+                e = int(idx[t, k])
+                want[t] += s[t, k] * (x[t] @ wup[e] @ wd[e])
+            if shared is not None:
+                want[t] += (x[t] @ sh[0] @ sh[1]) * torch.sigmoid(x[t] @ sh[2])
+        assert torch.allclose(res["y"], want, atol=1e-12)
+        assert res["inter"].shape == (T * K, I) and torch.equal(res["inter"], res["gate_up"])
+    # the gated layer on the same shapes is a different function (the activation is really absent above)
+    gated = O.forward(x, wr, torch.cat((wup, wup), dim=-1), wd, O.OracleConfig(H, I, E, K))
+    assert not torch.allclose(gated["y"], O.forward(x, wr, wup, wd, cfg)["y"], atol=1e-3)
+
+
 def test_whole_layer_with_shared_expert_against_hf_block():
     """The installed transformers Qwen2-MoE block = routed experts + shared MLP times a sigmoid
     gate (the block the reference's shared-expert parameters are filled from, utils.py:268-289)."""
