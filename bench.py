@@ -161,9 +161,13 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0)
     ap.add_argument("--kernel-iters", type=int, default=10)
+    ap.add_argument("--no-unragged", action="store_true",
+                    help="skip the yardstick's run of the dominant kernel on the un-ragged problem (a kernel trace "
+                         "averages per kernel symbol: this keeps its launches to the real problem)")
     ap.add_argument("--only-kernels", action="store_true",
-                    help="skip the timed layer steps, the yardstick and the CPU baseline: run each kernel --kernel-iters "
-                         "times (for counter collection), preceded by one plain 1 GiB device copy as a traffic yardstick")
+                    help="skip the timed layer steps and the CPU baseline: run each kernel (and the library GEMM of the "
+                         "yardstick) --kernel-iters times untimed, for counter collection, preceded by one plain 1 GiB "
+                         "device copy as a traffic yardstick")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the expert layer on ONE GPU; --gpus must be 1 (no multi-GPU path in this build)")
@@ -405,30 +409,61 @@ def main():
     for e_ in breakdown:
         e_.pop("_flops"), e_.pop("_bytes")
 
-    # ------------------------------------------------------------------ same-box yardstick: the library GEMM
+    # ------------------------------------------------------------------ same-box yardsticks
+    # (1) the library GEMM (torch.matmul -> hipBLASLt) on the dense equivalents of the dominant
+    # kernel's launches; (2) the dominant kernel itself on the un-ragged equivalent of its problem:
+    # every expert the same number of rows, no gather.  (2) / (1) is what the tile loop and its
+    # epilogue cost against the library, kernel / (2) what ragged expert loads and the gather cost.
+    # With --only-kernels (1) runs --kernel-iters times untimed, so that a counter pass sees the library's kernel too.
     yardstick = None
-    if dg["flops"] and not args.only_kernels and dtype == torch.bfloat16:
+    if dg["flops"] and dtype == torch.bfloat16:
         del gu, inter, out, d_inter, d_gu, d_xp
         torch.cuda.empty_cache()
-        y_ms = y_flops = 0.0
+        run = (lambda fn: [fn() for _ in range(it)] and 0.0) if args.only_kernels else (lambda fn: time_op(fn, it, torch))
+        y_ms = y_flops = u_ms = 0.0
         shapes = []
+        per = R // E
+        offs_u = torch.arange(E + 1, dtype=torch.int64) * per
+        offs_u[E] = R
+        offs_u = offs_u.to(torch.int32).to(dev)
+        rnd = lambda *shape: torch.randn(shape, device=dev, dtype=dtype)
         for m_ in dg["members"]:
             M_, K_, N_, lay = dense[m_]
-            a_ = torch.randn((K_, M_) if lay == "tn" else (M_, K_), device=dev, dtype=dtype)
-            b_ = torch.randn((N_, K_) if lay == "nt" else (K_, N_), device=dev, dtype=dtype) * 0.02
+            a_ = rnd(K_, M_) if lay == "tn" else rnd(M_, K_)
+            b_ = (rnd(N_, K_) if lay == "nt" else rnd(K_, N_)) * 0.02
             fn = {"nn": lambda: torch.matmul(a_, b_), "nt": lambda: torch.matmul(a_, b_.t()),
                   "tn": lambda: torch.matmul(a_.t(), b_)}[lay]
-            y_ms += time_op(fn, it, torch)
+            y_ms += run(fn)
             y_flops += 2.0 * M_ * K_ * N_
             shapes.append(f"{lay} {M_}x{K_}x{N_}")
             del a_, b_
-        y_tf = y_flops / (y_ms * 1e-3) / 1e12
-        yardstick = {
-            "what": "torch.matmul (hipBLASLt) on the dense, un-ragged equivalents of the dominant kernel's launches, same "
-                    "event timing, random data of the same distribution",
-            "shapes": shapes, "tflops": round(y_tf, 1), "frac_mfma_peak": round(y_tf / peak, 4),
-            "kernel_vs_yardstick": round(ach / y_tf, 4),
-        }
+            ufn = {
+                "gemm_gateup_act_fwd": lambda a: ops.grouped_gemm_gateup_act_fwd(a[0], wgu_d, offs_u, row_scale=s_perm, tile_cfg=c),
+                "gemm_down_fwd": lambda a: ops.grouped_gemm_nn(a[1], wd_d, offs_u, tile_cfg=c),
+                "gemm_dgrad_down": lambda a: ops.grouped_gemm_nt(a[0], wd_d, offs_u, tile_cfg=c),
+                "gemm_dgrad_down_gated_bwd": lambda a: ops.grouped_gemm_nt_gated_bwd(a[0], wd_d, offs_u, a[2], row_scale=s_perm,
+                                                                                      tile_cfg=c),
+                "gemm_dgrad_gateup": lambda a: ops.grouped_gemm_nt(a[2], wgu_d, offs_u, tile_cfg=c),
+                "gemm_wgrad_down": lambda a: ops.grouped_gemm_wgrad(a[1], a[0], offs_u, E, tile_cfg=c),
+                "gemm_wgrad_gateup": lambda a: ops.grouped_gemm_wgrad(a[0], a[2], offs_u, E, tile_cfg=c),
+            }[m_]
+            if not (args.only_kernels or args.no_unragged):  # (a profile averages per kernel symbol)
+                bufs = (rnd(R, H), rnd(R, I), rnd(R, 2 * I))   # rows of width H, I and 2I
+                u_ms += run(lambda: ufn(bufs))
+                del bufs
+        if not args.only_kernels:
+            y_tf = y_flops / (y_ms * 1e-3) / 1e12
+            u_tf = dg["flops"] / (u_ms * 1e-3) / 1e12 if u_ms else None
+            yardstick = {
+                "what": "torch.matmul (hipBLASLt) on the dense equivalents of the dominant kernel's launches, and that kernel "
+                        "on the un-ragged equivalent of its own problem (every expert R/E rows, no gather); same event "
+                        "timing, random data of the same distribution",
+                "shapes": shapes, "tflops": round(y_tf, 1), "frac_mfma_peak": round(y_tf / peak, 4),
+                "kernel_vs_yardstick": round(ach / y_tf, 4),
+            }
+            if u_tf:
+                yardstick.update(kernel_unragged_tflops=round(u_tf, 1), kernel_unragged_frac_mfma_peak=round(u_tf / peak, 4),
+                                 kernel_unragged_vs_yardstick=round(u_tf / y_tf, 4))
 
     result = {
         "metric": "moe_layer_fwd_bwd_tokens_per_s",
