@@ -35,6 +35,8 @@ static inline int amoe_check_launch(const char* what)
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16_t;
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
@@ -58,6 +60,15 @@ __device__ __forceinline__ float round_bf16(float a)
 {
     bf16_t r = (bf16_t)a;
     return (float)r;
+}
+
+// the same for IEEE half precision (v_cvt_f16_f32 rounds to nearest even in the default mode)
+__device__ __forceinline__ float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2_t, w)[0]; }
+__device__ __forceinline__ float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2_t, w)[1]; }
+__device__ __forceinline__ uint32_t pack_f16x2(float a, float b)
+{
+    f16x2_t r = {(f16_t)a, (f16_t)b};
+    return __builtin_bit_cast(uint32_t, r);
 }
 
 template <typename T>
@@ -103,6 +114,35 @@ struct ElemTraits<bf16_t> {
     __device__ static __forceinline__ void store1(bf16_t* p, float v) { *p = (bf16_t)v; }
     __device__ static __forceinline__ float round(float v) { return round_bf16(v); }
 };
+
+template <>
+struct ElemTraits<f16_t> {
+    static constexpr int kVec = 8;
+    __device__ static __forceinline__ void unpack(const u32x4_t& v, float* f)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = f16_lo(v[i]);
+            f[2 * i + 1] = f16_hi(v[i]);
+        }
+    }
+    __device__ static __forceinline__ u32x4_t pack(const float* f)
+    {
+        u32x4_t v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = pack_f16x2(f[2 * i], f[2 * i + 1]);
+        return v;
+    }
+    __device__ static __forceinline__ float load1(const f16_t* p) { return (float)(*p); }
+    __device__ static __forceinline__ void store1(f16_t* p, float v) { *p = (f16_t)v; }
+    __device__ static __forceinline__ float round(float v) { return (float)(f16_t)v; }
+};
+
+// runs the statement with ELEM = the element type of `dtype` (float for AMOE_F32)
+#define AMOE_DISPATCH_ELEM(dtype, ...)                                   \
+    if ((dtype) == AMOE_BF16) { typedef bf16_t ELEM; __VA_ARGS__; }      \
+    else if ((dtype) == AMOE_F16) { typedef f16_t ELEM; __VA_ARGS__; }   \
+    else { typedef float ELEM; __VA_ARGS__; }
 
 // Wave-wide reductions without LDS traffic: four DPP steps leave every lane of a 16-lane row
 // with the row's result (lanes exchanged inside quads, then between the quads of a half row,

@@ -35,7 +35,36 @@
 #include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 mfma_bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 mfma_f16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float mfma_f32x16;
+
+// What the kernel needs to know about its 16-bit element type: the MFMA operand vector and
+// instruction, and the conversions of the epilogues (round to nearest even on the way out).
+// Addresses, tiles and the LDS layout only depend on the element size, which the two types share.
+template <typename ET>
+struct Elem16;
+template <>
+struct Elem16<bf16_t> {
+    typedef mfma_bf16x8 frag_t;
+    __device__ static __forceinline__ float lo(uint32_t w) { return bf16_lo(w); }
+    __device__ static __forceinline__ float hi(uint32_t w) { return bf16_hi(w); }
+    __device__ static __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
+    __device__ static __forceinline__ mfma_f32x16 mfma(frag_t a, frag_t b, mfma_f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Elem16<f16_t> {
+    typedef mfma_f16x8 frag_t;
+    __device__ static __forceinline__ float lo(uint32_t w) { return f16_lo(w); }
+    __device__ static __forceinline__ float hi(uint32_t w) { return f16_hi(w); }
+    __device__ static __forceinline__ uint32_t pack2(float a, float b) { return pack_f16x2(a, b); }
+    __device__ static __forceinline__ mfma_f32x16 mfma(frag_t a, frag_t b, mfma_f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
 
 namespace {
 
@@ -69,6 +98,7 @@ struct GemmArgs {
     int gm, gn;   // blocks of one XCD work on super-tiles of gm x gn tiles
     int sn;       // super-tiles along N
     int max_mtiles;  // rows mode: entries of tile_map (those past the last tile hold expert -1)
+    int f16;         // host side only: the operands are float16 (launch the f16 instance), else bf16
 };
 
 enum { EPI_STORE = 0, EPI_GATED = 1, EPI_GATED_BWD = 2 };
@@ -183,10 +213,11 @@ using T_ = std::true_type;
 using F_ = std::false_type;
 
 // MAPS (weight gradient only): 1 = the rows of A, 2 = the rows of B are gathered through a row map
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
-__global__ void __launch_bounds__(WGM * WGN * 64)
-grouped_gemm_bf16_kernel(GemmArgs p)
+// ET: the 16-bit element type (bf16_t or f16_t); GemmArgs names its pointers bf16_t for both
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS, typename ET>
+__device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
 {
+    typedef typename Elem16<ET>::frag_t frag_t;
     constexpr int NT = WGM * WGN * 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -418,7 +449,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
         asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "i"((ks * 16 + 4) * cpr * 16));
         return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
     };
-    auto read_a = [&](const u32x4_t* sa, auto KS, mfma_bf16x8 (&fa)[TM]) {
+    auto read_a = [&](const u32x4_t* sa, auto KS, frag_t (&fa)[TM]) {
         constexpr int ks = decltype(KS)::value;
 #pragma unroll
         for (int t = 0; t < TM; ++t) {
@@ -430,10 +461,10 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             } else {
                 r = read_tr(sa, std::integral_constant<int, BM / 8>{}, wm * WTM + t * 32, KS);
             }
-            fa[t] = __builtin_bit_cast(mfma_bf16x8, r);
+            fa[t] = __builtin_bit_cast(frag_t, r);
         }
     };
-    auto read_b = [&](const u32x4_t* sb, auto KS, mfma_bf16x8 (&fb)[TN]) {
+    auto read_b = [&](const u32x4_t* sb, auto KS, frag_t (&fb)[TN]) {
         constexpr int ks = decltype(KS)::value;
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
@@ -445,13 +476,13 @@ grouped_gemm_bf16_kernel(GemmArgs p)
             } else {
                 r = read_tr(sb, std::integral_constant<int, BN / 8>{}, wn * WTN + t * 32, KS);
             }
-            fb[t] = __builtin_bit_cast(mfma_bf16x8, r);
+            fb[t] = __builtin_bit_cast(frag_t, r);
         }
     };
     // Called before the first MFMA that consumes fragments fetched by read_tr: waits for this
     // wave's LDS reads and makes the fragments depend on the wait (an MFMA is otherwise free to
     // be scheduled ahead of it).
-    auto settle = [&](mfma_bf16x8 (&fa)[TM], mfma_bf16x8 (&fb)[TN]) {
+    auto settle = [&](frag_t (&fa)[TM], frag_t (&fb)[TN]) {
         if (A_KC && B_KC) return;
         asm volatile("s_waitcnt lgkmcnt(0)");
         if (!A_KC) {
@@ -466,12 +497,12 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     // quarter Q of a K step's MFMAs (A tile outer, B tile inner)
     constexpr int N_MFMA = TM * TN;
     static_assert(N_MFMA % 4 == 0, "a K step is issued in four chunks");
-    auto mma_quarter = [&](const mfma_bf16x8 (&fa)[TM], const mfma_bf16x8 (&fb)[TN], auto Q) {
+    auto mma_quarter = [&](const frag_t (&fa)[TM], const frag_t (&fb)[TN], auto Q) {
         constexpr int q = decltype(Q)::value;
 #pragma unroll
         for (int f = q * (N_MFMA / 4); f < (q + 1) * (N_MFMA / 4); ++f) {
             const int i = f / TN, j = f % TN;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            acc[i][j] = Elem16<ET>::mfma(fa[i], fb[j], acc[i][j]);
         }
     };
 
@@ -499,7 +530,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
     using A_ALL = std::integral_constant<int, PER_A>;
     using B_HALF = std::integral_constant<int, (PER_B + 1) / 2>;
     using B_ALL = std::integral_constant<int, PER_B>;
-    mfma_bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    frag_t fa0[TM], fb0[TN], fa1[TM], fb1[TN];
 
     // prologue: tiles 0..2 and the A half of tile 3 go out, tile 0 is awaited
     {
@@ -654,12 +685,12 @@ grouped_gemm_bf16_kernel(GemmArgs p)
                     float h[2];
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
-                        const uint32_t own = pack_bf16x2(acc[i][j][v + 2 * u], acc[i][j][v + 2 * u + 1]);
+                        const uint32_t own = Elem16<ET>::pack2(acc[i][j][v + 2 * u], acc[i][j][v + 2 * u + 1]);
                         const uint32_t got = __builtin_amdgcn_update_dpp(0, own, 0xB1, 0xF, 0xF, true);
                         const uint32_t pk = __builtin_amdgcn_perm(got, own, swap_sel);
                         const bool ok = full || (col_ok && m0 + rt + 2 * u + odd1 < mend);
                         if (EPI == EPI_GATED)
-                            h[u] = sc[v >> 2][u] * bf16_hi(pk) * act_fwd_fast<ACT>(bf16_lo(pk));
+                            h[u] = sc[v >> 2][u] * Elem16<ET>::hi(pk) * act_fwd_fast<ACT>(Elem16<ET>::lo(pk));
                         if (want_c && ok) {
                             char* rowp = cbase + ((long long)(rq + 2 * u) * p.ldc + j * 32) * 2;
                             *reinterpret_cast<uint32_t*>(rowp + loff) = pk;
@@ -668,7 +699,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
                     if (EPI == EPI_GATED) {
                         // lanes with bit 1 clear keep the first row pair, the others the second
                         const float got = lane_xor2(odd2 ? h[0] : h[1]);
-                        const uint32_t hp = odd2 ? pack_bf16x2(got, h[1]) : pack_bf16x2(h[0], got);
+                        const uint32_t hp = odd2 ? Elem16<ET>::pack2(got, h[1]) : Elem16<ET>::pack2(h[0], got);
                         const bool ok = full || (col_ok && m0 + rt + 2 * odd2 + odd1 < mend);
                         if (ok) {
                             char* rowp = c2base + ((long long)rq * p.ldc2 + j * 16) * 2;
@@ -731,7 +762,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
                         const int v = 8 * hh + u;
                         const int rr = i * 32 + 8 * (v >> 2) + (v & 3);
                         const float d = acc[i][j][v];
-                        const float gate = bf16_lo(gcur[u]), up = bf16_hi(gcur[u]);
+                        const float gate = Elem16<ET>::lo(gcur[u]), up = Elem16<ET>::hi(gcur[u]);
                         float f, df;
                         act_both_fast<ACT>(gate, f, df);
                         const float sd = s_rs[wm * WTM + rr + 4 * lg] * d;
@@ -739,7 +770,7 @@ grouped_gemm_bf16_kernel(GemmArgs p)
                         const bool ok = full || (col_ok && m0 + wm * WTM + rr + 4 * lg < mend);
                         if (ok) {
                             char* rowp = dbase + ((long long)rr * p.ldg + 2 * j * 32) * 2;
-                            *reinterpret_cast<uint32_t*>(rowp + goff) = pack_bf16x2(sd * up * df, sd * f);
+                            *reinterpret_cast<uint32_t*>(rowp + goff) = Elem16<ET>::pack2(sd * up * df, sd * f);
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);
@@ -780,27 +811,57 @@ grouped_gemm_bf16_kernel(GemmArgs p)
 }
 
 // ------------------------------------------------------------------ host side
+
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
-int launch_cfg(const GemmArgs& a, int grid, hipStream_t s)
+__global__ void __launch_bounds__(WGM * WGN * 64)
+grouped_gemm_bf16_kernel(GemmArgs p)
 {
-    auto kern = grouped_gemm_bf16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS>;
-    constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
+    grouped_gemm_body<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS, bf16_t>(p);
+}
+
+// the same kernel on float16 operands (v_mfma_f32_32x32x16_f16)
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
+__global__ void __launch_bounds__(WGM * WGN * 64)
+grouped_gemm_f16_kernel(GemmArgs p)
+{
+    grouped_gemm_body<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS, f16_t>(p);
+}
+
+template <auto KERN, int THREADS, int LDS_BYTES>
+int launch_kernel(const GemmArgs& a, int grid, hipStream_t s)
+{
     // The LDS limit is an attribute of the kernel on one device: set once per device (bit d of the
     // mask); setting it twice from racing threads is harmless.
     static std::atomic<unsigned long long> attr_done{0};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 63;   // 63: never cached
     if (dev == 63 || !(attr_done.load(std::memory_order_relaxed) >> dev & 1ull)) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(KERN),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (err != hipSuccess) {
-            amoe_set_error("grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(err));
+            amoe_set_error("grouped_gemm: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(err));
             return AMOE_ERR_LAUNCH;
         }
         if (dev != 63) attr_done.fetch_or(1ull << dev, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(WGM * WGN * 64), lds_bytes, s, a);
-    return amoe_check_launch("grouped_gemm_bf16");
+    hipLaunchKernelGGL(KERN, dim3(grid), dim3(THREADS), LDS_BYTES, s, a);
+    return amoe_check_launch("grouped_gemm_16bit");
+}
+
+// F16_OK = false leaves the float16 instance of this shape out of the library
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0, bool F16_OK = true>
+int launch_cfg(const GemmArgs& a, int grid, hipStream_t s)
+{
+    constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
+    if (a.f16) {
+        if constexpr (F16_OK) {
+            return launch_kernel<grouped_gemm_f16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS>, WGM * WGN * 64, lds_bytes>(a, grid, s);
+        } else {
+            amoe_set_error("grouped_gemm: this tile_cfg is not available for float16 with this epilogue");
+            return AMOE_ERR_UNSUPPORTED;
+        }
+    }
+    return launch_kernel<grouped_gemm_bf16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS>, WGM * WGN * 64, lds_bytes>(a, grid, s);
 }
 
 struct TileCfg {
@@ -830,7 +891,8 @@ int launch_any(const GemmArgs& a, int tile_cfg, int grid, hipStream_t s)
                 amoe_set_error("grouped_gemm: tile_cfg 3 is not available with the gated-backward epilogue");
                 return AMOE_ERR_UNSUPPORTED;
             } else {
-                return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT, MAPS>(a, grid, s);
+                // (the float16 conversions of the gated epilogue do not fit beside them either)
+                return launch_cfg<256, 256, 2, 2, A_KC, B_KC, EPI, ACT, MAPS, EPI != EPI_GATED>(a, grid, s);
             }
         case 5:
             if constexpr (EPI == EPI_GATED_BWD) {   // spills as well (four tile columns per wave)
@@ -897,7 +959,7 @@ int amoe_build_tile_map(const int32_t* offsets, int R, int E, int bm, void* work
 int amoe_tile_map_layout(int R, int E, int dtype, int tile_cfg, void* workspace, size_t workspace_bytes, int4** tile_map,
                          int32_t** n_mtiles, int* bm, int* max_mtiles)
 {
-    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "tile map: bad dtype %d", dtype);
+    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16 || dtype == AMOE_F16, AMOE_ERR_BAD_ARG, "tile map: bad dtype %d", dtype);
     const int shape = tile_cfg & ~AMOE_TILE_MAP_READY;
     AMOE_REQUIRE(tile_cfg >= 0 && shape <= 5 && shape != 4, AMOE_ERR_BAD_ARG, "tile map: bad tile_cfg %d", tile_cfg);
     AMOE_REQUIRE(R > 0 && E > 0 && E <= AMOE_MAX_EXPERTS, AMOE_ERR_BAD_ARG, "tile map: bad sizes R=%d E=%d", R, E);
@@ -914,7 +976,7 @@ int amoe_tile_map_layout(int R, int E, int dtype, int tile_cfg, void* workspace,
 template <bool B_KC, int EPI, int ACT>
 static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C,
                          void* C2, const float* row_scale, int R, int E, int Kred, int N, int ldb, long long strideB, void* workspace,
-                         size_t workspace_bytes, int tile_cfg, hipStream_t s, const void* G = nullptr, float* partials = nullptr)
+                         size_t workspace_bytes, int tile_cfg, hipStream_t s, int dtype, const void* G = nullptr, float* partials = nullptr)
 {
     const bool map_ready = (tile_cfg & AMOE_TILE_MAP_READY) != 0;
     tile_cfg &= ~AMOE_TILE_MAP_READY;
@@ -928,6 +990,7 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
     a.B = (const bf16_t*)B;
     a.C = (bf16_t*)C;
     a.C2 = (bf16_t*)C2;
+    a.f16 = dtype == AMOE_F16;
     a.a_row_map = a_row_map;
     a.row_scale = row_scale;
     a.offsets = offsets;
@@ -956,27 +1019,27 @@ static int run_rows_bf16(const void* A, const int32_t* a_row_map, const void* B,
 
 int amoe_bf16_gateup_act(const void* xp, const int32_t* a_row_map, const void* w, const int32_t* offsets, void* gate_up,
                          void* inter, const float* row_scale, int R, int E, int H, int I, int act, void* workspace, size_t workspace_bytes,
-                         int tile_cfg, hipStream_t s)
+                         int tile_cfg, hipStream_t s, int dtype)
 {
     AMOE_DISPATCH_ACT(act, return (run_rows_bf16<false, EPI_GATED, ACT>(xp, a_row_map, w, offsets, gate_up, inter, row_scale, R, E, H,
                                                                         2 * I, 2 * I, (long long)H * 2 * I, workspace,
-                                                                        workspace_bytes, tile_cfg, s)))
+                                                                        workspace_bytes, tile_cfg, s, dtype)))
     return AMOE_ERR_BAD_ARG;
 }
 
 int amoe_bf16_nn(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
-                 int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s)
+                 int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s, int dtype)
 {
     return run_rows_bf16<false, EPI_STORE, 0>(A, a_row_map, B, offsets, C, nullptr, nullptr, R, E, Kd, N, N, (long long)Kd * N,
-                                              workspace, workspace_bytes, tile_cfg, s);
+                                              workspace, workspace_bytes, tile_cfg, s, dtype);
 }
 
 // C[rows_e, :Kd] = A[rows_e, :N] @ B[e]^T with B [E, Kd, N]: the reduction runs over N
 int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
-                 int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s)
+                 int Kd, int N, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s, int dtype)
 {
     return run_rows_bf16<true, EPI_STORE, 0>(A, a_row_map, B, offsets, C, nullptr, nullptr, R, E, /*Kred=*/N, /*N out=*/Kd,
-                                             /*ldb=*/N, (long long)Kd * N, workspace, workspace_bytes, tile_cfg, s);
+                                             /*ldb=*/N, (long long)Kd * N, workspace, workspace_bytes, tile_cfg, s, dtype);
 }
 
 // d_gate_up [R, 2I] and the row sums of the score gradient from dy rows [., H], w_down [E, I, H] and the
@@ -984,12 +1047,12 @@ int amoe_bf16_nt(const void* A, const int32_t* a_row_map, const void* B, const i
 // activation as its epilogue.  The reduction runs over H, the output columns are the I intermediate columns.
 int amoe_bf16_nt_gated_bwd(const void* dy, const int32_t* a_row_map, const void* w_down, const int32_t* offsets,
                            const void* gate_up, const float* row_scale, void* d_gate_up, float* partials, int R, int E,
-                           int I, int H, int act, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s)
+                           int I, int H, int act, void* workspace, size_t workspace_bytes, int tile_cfg, hipStream_t s, int dtype)
 {
     AMOE_DISPATCH_ACT(act, return (run_rows_bf16<true, EPI_GATED_BWD, ACT>(dy, a_row_map, w_down, offsets, d_gate_up, nullptr,
                                                                            row_scale, R, E, /*Kred=*/H, /*N out=*/I, /*ldb=*/H,
                                                                            (long long)I * H, workspace, workspace_bytes,
-                                                                           tile_cfg, s, gate_up, partials)))
+                                                                           tile_cfg, s, dtype, gate_up, partials)))
     return AMOE_ERR_BAD_ARG;
 }
 
@@ -1001,11 +1064,12 @@ int amoe_bf16_gated_bwd_parts(int I, int tile_cfg)
 }
 
 int amoe_bf16_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
-                    const int32_t* offsets, void* C, int R, int E, int Kd, int N, int tile_cfg, hipStream_t s)
+                    const int32_t* offsets, void* C, int R, int E, int Kd, int N, int tile_cfg, hipStream_t s, int dtype)
 {
     tile_cfg &= ~AMOE_TILE_MAP_READY;   // no tile map in the weight gradient
     TileCfg tc = pick_cfg(tile_cfg);
     GemmArgs a = {};
+    a.f16 = dtype == AMOE_F16;
     a.A = (const bf16_t*)A;
     a.B = (const bf16_t*)B;
     a.C = (bf16_t*)C;

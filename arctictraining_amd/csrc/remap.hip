@@ -112,10 +112,10 @@ int launch(bool pack, const void* a0, const void* a1, void* b0, void* b1, int E,
 int check(const char* what, const void* p0, const void* p1, int dtype, int E, int I, int H, long long split_es)
 {
     AMOE_REQUIRE(p0 && p1, AMOE_ERR_BAD_ARG, "%s: null pointer", what);
-    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "%s: bad dtype %d", what, dtype);
+    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16 || dtype == AMOE_F16, AMOE_ERR_BAD_ARG, "%s: bad dtype %d", what, dtype);
     AMOE_REQUIRE(E > 0 && I > 0 && H > 0, AMOE_ERR_BAD_ARG, "%s: sizes must be positive (E=%d I=%d H=%d)", what, E, I, H);
     AMOE_REQUIRE(E <= 65535 && (I + TILE - 1) / TILE <= 65535, AMOE_ERR_UNSUPPORTED, "%s: grid too large", what);
-    const int v = dtype == AMOE_BF16 ? 8 : 4;
+    const int v = dtype != AMOE_F32 ? 8 : 4;
     AMOE_REQUIRE(I % v == 0 && H % v == 0, AMOE_ERR_UNSUPPORTED, "%s: I=%d and H=%d must be multiples of %d", what, I, H, v);
     AMOE_REQUIRE(split_es >= (long long)I * H && split_es % v == 0, AMOE_ERR_BAD_ARG,
                  "%s: expert stride %lld must be at least I*H and a multiple of %d", what, split_es, v);
@@ -129,7 +129,7 @@ AMOE_EXPORT int amoe_remap_pack(const void* in0, const void* in1, void* out, int
 {
     int rc = check("amoe_remap_pack", in0, out, dtype, E, I, H, in_expert_stride);
     if (rc) return rc;
-    if (dtype == AMOE_BF16) return launch<uint16_t>(true, in0, in1, out, nullptr, E, I, H, in_expert_stride, (hipStream_t)stream);
+    if (dtype != AMOE_F32) return launch<uint16_t>(true, in0, in1, out, nullptr, E, I, H, in_expert_stride, (hipStream_t)stream);
     return launch<uint32_t>(true, in0, in1, out, nullptr, E, I, H, in_expert_stride, (hipStream_t)stream);
 }
 
@@ -138,6 +138,6 @@ AMOE_EXPORT int amoe_remap_unpack(const void* in, void* out0, void* out1, int dt
 {
     int rc = check("amoe_remap_unpack", in, out0, dtype, E, I, H, out_expert_stride);
     if (rc) return rc;
-    if (dtype == AMOE_BF16) return launch<uint16_t>(false, in, nullptr, out0, out1, E, I, H, out_expert_stride, (hipStream_t)stream);
+    if (dtype != AMOE_F32) return launch<uint16_t>(false, in, nullptr, out0, out1, E, I, H, out_expert_stride, (hipStream_t)stream);
     return launch<uint32_t>(false, in, nullptr, out0, out1, E, I, H, out_expert_stride, (hipStream_t)stream);
 }

@@ -62,7 +62,8 @@ __device__ __forceinline__ uint32_t wave_max_key(uint32_t k)
     return ab > cd ? ab : cd;
 }
 
-// key type, construction and index extraction per logit type
+// key type, construction and index extraction per logit type (float16 logits take the 64-bit key:
+// their 11 significant bits do not fit the upper half of the float32 pattern)
 template <typename T>
 struct SelKey {
     typedef unsigned long long type;
@@ -248,18 +249,14 @@ AMOE_EXPORT int amoe_router_topk_fwd(const void* logits, int dtype, int T, int E
                                      int32_t* topk_idx, float* scores, void* stream)
 {
     AMOE_REQUIRE(logits && probs && topk_idx && scores, AMOE_ERR_BAD_ARG, "router_topk_fwd: null pointer");
-    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "router_topk_fwd: bad dtype %d", dtype);
+    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16 || dtype == AMOE_F16, AMOE_ERR_BAD_ARG, "router_topk_fwd: bad dtype %d", dtype);
     int rc = check_router_shape(T, E, K);
     if (rc) return rc;
     dim3 grid((T + kTokensPerBlock - 1) / kTokensPerBlock), block(kTokensPerBlock * AMOE_WAVE);
     hipStream_t s = (hipStream_t)stream;
     ROUTER_DISPATCH_VPT(E, {
-        if (dtype == AMOE_BF16)
-            hipLaunchKernelGGL((router_topk_fwd_kernel<bf16_t, VPT>), grid, block, 0, s, (const bf16_t*)logits, T, E, K,
-                               normalize, probs, topk_idx, scores);
-        else
-            hipLaunchKernelGGL((router_topk_fwd_kernel<float, VPT>), grid, block, 0, s, (const float*)logits, T, E, K,
-                               normalize, probs, topk_idx, scores);
+        AMOE_DISPATCH_ELEM(dtype, hipLaunchKernelGGL((router_topk_fwd_kernel<ELEM, VPT>), grid, block, 0, s,
+                                                     (const ELEM*)logits, T, E, K, normalize, probs, topk_idx, scores))
     })
     return amoe_check_launch("router_topk_fwd");
 }
@@ -269,18 +266,14 @@ AMOE_EXPORT int amoe_router_bwd(const float* d_scores, const float* probs, const
                                 void* d_logits, void* stream)
 {
     AMOE_REQUIRE(d_scores && probs && topk_idx && counts && d_logits, AMOE_ERR_BAD_ARG, "router_bwd: null pointer");
-    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "router_bwd: bad dtype %d", dtype);
+    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16 || dtype == AMOE_F16, AMOE_ERR_BAD_ARG, "router_bwd: bad dtype %d", dtype);
     int rc = check_router_shape(T, E, K);
     if (rc) return rc;
     dim3 grid((T + kTokensPerBlock - 1) / kTokensPerBlock), block(kTokensPerBlock * AMOE_WAVE);
     hipStream_t s = (hipStream_t)stream;
     ROUTER_DISPATCH_VPT(E, {
-        if (dtype == AMOE_BF16)
-            hipLaunchKernelGGL((router_bwd_kernel<bf16_t, VPT>), grid, block, 0, s, d_scores, probs, topk_idx, counts, T,
-                               E, K, normalize, lb_coeff, (bf16_t*)d_logits);
-        else
-            hipLaunchKernelGGL((router_bwd_kernel<float, VPT>), grid, block, 0, s, d_scores, probs, topk_idx, counts, T,
-                               E, K, normalize, lb_coeff, (float*)d_logits);
+        AMOE_DISPATCH_ELEM(dtype, hipLaunchKernelGGL((router_bwd_kernel<ELEM, VPT>), grid, block, 0, s, d_scores, probs,
+                                                     topk_idx, counts, T, E, K, normalize, lb_coeff, (ELEM*)d_logits))
     })
     return amoe_check_launch("router_bwd");
 }

@@ -195,9 +195,9 @@ score_grad_gather_kernel(const float* __restrict__ partials, int n_parts, long l
 
 int check_rows(const char* what, int dtype, int rows, int H)
 {
-    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16, AMOE_ERR_BAD_ARG, "%s: bad dtype %d", what, dtype);
+    AMOE_REQUIRE(dtype == AMOE_F32 || dtype == AMOE_BF16 || dtype == AMOE_F16, AMOE_ERR_BAD_ARG, "%s: bad dtype %d", what, dtype);
     AMOE_REQUIRE(rows > 0 && H > 0, AMOE_ERR_BAD_ARG, "%s: sizes must be positive (rows=%d H=%d)", what, rows, H);
-    const int vec = dtype == AMOE_BF16 ? 8 : 4;
+    const int vec = dtype != AMOE_F32 ? 8 : 4;
     AMOE_REQUIRE(H % vec == 0, AMOE_ERR_UNSUPPORTED, "%s: row length %d must be a multiple of %d", what, H, vec);
     return AMOE_OK;
 }
@@ -213,12 +213,8 @@ AMOE_EXPORT int amoe_gather_rows_fwd(const void* x, const int32_t* token_of, voi
     int rc = check_rows("gather_rows_fwd", dtype, R, H);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == AMOE_BF16)
-        hipLaunchKernelGGL(gather_rows_kernel<bf16_t>, dim3(row_grid(R)), dim3(kBlock), 0, s, (const bf16_t*)x, token_of,
-                           (bf16_t*)xp, R, H);
-    else
-        hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(row_grid(R)), dim3(kBlock), 0, s, (const float*)x, token_of,
-                           (float*)xp, R, H);
+    AMOE_DISPATCH_ELEM(dtype, hipLaunchKernelGGL(gather_rows_kernel<ELEM>, dim3(row_grid(R)), dim3(kBlock), 0, s,
+                                                 (const ELEM*)x, token_of, (ELEM*)xp, R, H))
     return amoe_check_launch("gather_rows_fwd");
 }
 
@@ -249,10 +245,7 @@ AMOE_EXPORT int amoe_gather_rows_bwd(const void* d_xp, const int32_t* row_of, co
     if (rc) return rc;
     AMOE_REQUIRE(K > 0 && K <= AMOE_MAX_TOPK, AMOE_ERR_UNSUPPORTED, "gather_rows_bwd: K=%d outside 1..%d", K,
                  AMOE_MAX_TOPK);
-    if (dtype == AMOE_BF16)
-        launch_gather_reduce<bf16_t>(d_xp, row_of, nullptr, addend, dx, T, K, H, (hipStream_t)stream);
-    else
-        launch_gather_reduce<float>(d_xp, row_of, nullptr, addend, dx, T, K, H, (hipStream_t)stream);
+    AMOE_DISPATCH_ELEM(dtype, launch_gather_reduce<ELEM>(d_xp, row_of, nullptr, addend, dx, T, K, H, (hipStream_t)stream))
     return amoe_check_launch("gather_rows_bwd");
 }
 
@@ -263,10 +256,7 @@ AMOE_EXPORT int amoe_combine_fwd(const void* moe_out, const int32_t* row_of, con
     int rc = check_rows("combine_fwd", dtype, T, H);
     if (rc) return rc;
     AMOE_REQUIRE(K > 0 && K <= AMOE_MAX_TOPK, AMOE_ERR_UNSUPPORTED, "combine_fwd: K=%d outside 1..%d", K, AMOE_MAX_TOPK);
-    if (dtype == AMOE_BF16)
-        launch_gather_reduce<bf16_t>(moe_out, row_of, scores, nullptr, y, T, K, H, (hipStream_t)stream);
-    else
-        launch_gather_reduce<float>(moe_out, row_of, scores, nullptr, y, T, K, H, (hipStream_t)stream);
+    AMOE_DISPATCH_ELEM(dtype, launch_gather_reduce<ELEM>(moe_out, row_of, scores, nullptr, y, T, K, H, (hipStream_t)stream))
     return amoe_check_launch("combine_fwd");
 }
 
@@ -278,12 +268,9 @@ AMOE_EXPORT int amoe_combine_bwd(const void* dy, const void* moe_out, const int3
     if (rc) return rc;
     AMOE_REQUIRE(K > 0 && K <= AMOE_MAX_TOPK, AMOE_ERR_UNSUPPORTED, "combine_bwd: K=%d outside 1..%d", K, AMOE_MAX_TOPK);
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == AMOE_BF16)
-        hipLaunchKernelGGL(combine_bwd_kernel<bf16_t>, dim3(row_grid(T)), dim3(kBlock), 0, s, (const bf16_t*)dy,
-                           (const bf16_t*)moe_out, row_of, scores, (bf16_t*)d_moe_out, d_scores, T, K, H);
-    else
-        hipLaunchKernelGGL(combine_bwd_kernel<float>, dim3(row_grid(T)), dim3(kBlock), 0, s, (const float*)dy,
-                           (const float*)moe_out, row_of, scores, (float*)d_moe_out, d_scores, T, K, H);
+    AMOE_DISPATCH_ELEM(dtype, hipLaunchKernelGGL(combine_bwd_kernel<ELEM>, dim3(row_grid(T)), dim3(kBlock), 0, s,
+                                                 (const ELEM*)dy, (const ELEM*)moe_out, row_of, scores, (ELEM*)d_moe_out,
+                                                 d_scores, T, K, H))
     return amoe_check_launch("combine_bwd");
 }
 
@@ -294,12 +281,8 @@ int amoe_launch_gated_act_fwd(const void* gu, const float* row_scale, void* inte
     const int rows_per_block = kBlock / AMOE_WAVE;
     const int grid = (R + rows_per_block - 1) / rows_per_block < 65536 ? (R + rows_per_block - 1) / rows_per_block : 65536;
     AMOE_DISPATCH_ACT(act, {
-        if (dtype == AMOE_BF16)
-            hipLaunchKernelGGL((gated_act_fwd_kernel<bf16_t, ACT>), dim3(grid), dim3(kBlock), 0, s, (const bf16_t*)gu,
-                               row_scale, (bf16_t*)inter, R, I);
-        else
-            hipLaunchKernelGGL((gated_act_fwd_kernel<float, ACT>), dim3(grid), dim3(kBlock), 0, s, (const float*)gu,
-                               row_scale, (float*)inter, R, I);
+        AMOE_DISPATCH_ELEM(dtype, hipLaunchKernelGGL((gated_act_fwd_kernel<ELEM, ACT>), dim3(grid), dim3(kBlock), 0, s,
+                                                     (const ELEM*)gu, row_scale, (ELEM*)inter, R, I))
     })
     return amoe_check_launch("gated_act_fwd");
 }
@@ -322,13 +305,9 @@ AMOE_EXPORT int amoe_gated_act_bwd(const void* gate_up, const void* d_inter, con
     const int grid = (R + rows_per_block - 1) / rows_per_block < 65536 ? (R + rows_per_block - 1) / rows_per_block : 65536;
     hipStream_t s = (hipStream_t)stream;
     AMOE_DISPATCH_ACT(act, {
-        if (dtype == AMOE_BF16)
-            hipLaunchKernelGGL((gated_act_bwd_kernel<bf16_t, ACT>), dim3(grid), dim3(kBlock), 0, s,
-                               (const bf16_t*)gate_up, (const bf16_t*)d_inter, row_scale, slot_of, T, K,
-                               (bf16_t*)d_gate_up, d_row_scale, R, I);
-        else
-            hipLaunchKernelGGL((gated_act_bwd_kernel<float, ACT>), dim3(grid), dim3(kBlock), 0, s, (const float*)gate_up,
-                               (const float*)d_inter, row_scale, slot_of, T, K, (float*)d_gate_up, d_row_scale, R, I);
+        AMOE_DISPATCH_ELEM(dtype, hipLaunchKernelGGL((gated_act_bwd_kernel<ELEM, ACT>), dim3(grid), dim3(kBlock), 0, s,
+                                                     (const ELEM*)gate_up, (const ELEM*)d_inter, row_scale, slot_of, T, K,
+                                                     (ELEM*)d_gate_up, d_row_scale, R, I))
     })
     return amoe_check_launch("gated_act_bwd");
 }

@@ -144,7 +144,7 @@ def _dense_weight_grad(a: torch.Tensor, b: torch.Tensor, tile_cfg: int = 0, tile
     T, Kd = a.shape
     N = b.shape[1]
     tiles = -(-Kd // tile) * -(-N // tile)
-    splits = max(1, min(16, 512 // tiles, T // 256)) if a.dtype == torch.bfloat16 else 1
+    splits = max(1, min(16, 512 // tiles, T // 256)) if a.dtype != torch.float32 else 1
     part = ops.grouped_gemm_wgrad(a, b, _token_offsets(T, splits, a.device), splits, tile_cfg=tile_cfg)
     if splits == 1:
         return part[0]
@@ -155,7 +155,7 @@ def _router_weight_grad(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor
     """dW_router [E,H] = d_logits^T [E,T] @ x [T,H] (autograd of moe.py:233): skinny (E rows) and
     deep (T), the library GEMM leaves most of the chip idle on it."""
     T, E = d_logits.shape
-    if x.dtype != torch.bfloat16 or E % 8 or T < 16 * 32:
+    if x.dtype == torch.float32 or E % 8 or T < 16 * 32:
         return torch.matmul(d_logits.t(), x)
     return _dense_weight_grad(d_logits, x, tile_cfg=1, tile=128)  # 128x128 tiles
 
@@ -273,7 +273,7 @@ class _ExpertLayerFn(torch.autograd.Function):
 
         # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMMs' loads
         ws = ctx.gemm_ws  # still holds the forward's tile map
-        fused = x.dtype == torch.bfloat16 and cfg in (0, 1, 2)
+        fused = x.dtype != torch.float32 and cfg in (0, 1, 2)
         if fused:
             # data gradient of the down projection with the gated-activation backward as its
             # epilogue: d_inter is never written; the score gradients come back as per-N-tile row sums

@@ -9,17 +9,19 @@ import torch
 
 from . import _lib
 
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
+_DTYPE_CODES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 ACT_SILU, ACT_GELU, ACT_RELU, ACT_GPT_OSS = 0, 1, 2, 3
 TILE_MAP_READY = 0x100  # AMOE_TILE_MAP_READY
 
 
-def _dtype_code(t: torch.Tensor) -> int:
-    if t.dtype == torch.float32:
-        return F32
-    if t.dtype == torch.bfloat16:
-        return BF16
-    raise RuntimeError(f"the expert-layer kernels support float32 and bfloat16, not {t.dtype}")
+def _dtype_code(t) -> int:
+    """dtype code of the C ABI for a tensor or a torch dtype"""
+    dt = t.dtype if isinstance(t, torch.Tensor) else t
+    code = _DTYPE_CODES.get(dt)
+    if code is None:
+        raise RuntimeError(f"the expert-layer kernels support float32, bfloat16 and float16, not {dt}")
+    return code
 
 
 def _chk(t: torch.Tensor, name: str, dtype=None) -> torch.Tensor:
@@ -102,7 +104,7 @@ def permute_plan(assign: torch.Tensor, num_experts: int, scores: Optional[torch.
         rc = lib.amoe_permute_plan_tiled(
             assign.data_ptr(), _ptr(scores), T, K, E, counts.data_ptr(), offsets.data_ptr(), token_of.data_ptr(),
             slot_of.data_ptr(), row_of.data_ptr(), _ptr(scores_perm), ws.data_ptr(), ws.numel(), gemm_workspace.data_ptr(),
-            gemm_workspace.numel(), F32 if gemm_dtype == torch.float32 else BF16, tile_cfg, _stream()
+            gemm_workspace.numel(), _dtype_code(gemm_dtype), tile_cfg, _stream()
         )
         _lib.check(rc, "amoe_permute_plan_tiled")
         return counts, offsets, token_of, slot_of, row_of, scores_perm
@@ -298,9 +300,11 @@ def grouped_gemm_nt_gated_bwd(dy, w_down, offsets, gate_up, act: int = ACT_SILU,
     (gathered through a_row_map), w_down [E,I,H] and the forward's gate_up [R,2I]: the data gradient
     of the down projection with the gated-activation backward as its epilogue (bf16 only)."""
     lib = _lib.load()
-    _chk(dy, "dy", torch.bfloat16)
-    _chk(w_down, "w_down", torch.bfloat16)
-    _chk(gate_up, "gate_up", torch.bfloat16)
+    if dy.dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError("grouped_gemm_nt_gated_bwd: bfloat16 or float16 operands only")
+    _chk(dy, "dy")
+    _chk(w_down, "w_down", dy.dtype)
+    _chk(gate_up, "gate_up", dy.dtype)
     _chk(offsets, "offsets", torch.int32)
     if a_row_map is not None:
         _chk(a_row_map, "a_row_map", torch.int32)
@@ -317,7 +321,7 @@ def grouped_gemm_nt_gated_bwd(dy, w_down, offsets, gate_up, act: int = ACT_SILU,
     ws, tile_cfg = _ws_and_cfg(R, E, dy.device, tile_cfg, workspace, map_ready)
     rc = lib.amoe_grouped_gemm_nt_gated_bwd(
         dy.data_ptr(), _ptr(a_row_map), w_down.data_ptr(), offsets.data_ptr(), gate_up.data_ptr(), _ptr(row_scale),
-        d_gate_up.data_ptr(), _ptr(parts), BF16, R, E, I, H, act, ws.data_ptr(), ws.numel(), tile_cfg, _stream()
+        d_gate_up.data_ptr(), _ptr(parts), _dtype_code(dy), R, E, I, H, act, ws.data_ptr(), ws.numel(), tile_cfg, _stream()
     )
     _lib.check(rc, "amoe_grouped_gemm_nt_gated_bwd")
     return d_gate_up, parts

@@ -13,7 +13,9 @@
  *   - return 0 on success or a negative AMOE_ERR_* code; arguments are validated before
  *     the first HIP call, so argument errors can be exercised without a GPU;
  *     amoe_last_error() returns the calling thread's last message;
- *   - dtype: AMOE_F32 or AMOE_BF16 for activations / weights; probabilities, scores and
+ *   - dtype: AMOE_F32, AMOE_BF16 or AMOE_F16 for activations / weights (the three types the
+ *     reference's kernels dispatch, top_k_gating.cpp:56-59; the two 16-bit types share one
+ *     kernel apart from the matrix instruction and the conversions); probabilities, scores and
  *     score gradients are always float32; indices are int32 (routed rows R = T*K < 2^31);
  *   - routed-row order is the reference's (moe.py:367-382): grouped by expert ascending,
  *     inside an expert ascending flat slot f = k*T + t.
@@ -36,6 +38,7 @@ extern "C" {
 
 #define AMOE_F32 0
 #define AMOE_BF16 1
+#define AMOE_F16 2 /* IEEE half precision */
 
 #define AMOE_ACT_SILU 0
 #define AMOE_ACT_GELU 1
@@ -206,7 +209,7 @@ int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, const void* B,
  * the forward pass, row_scale [R] f32 or null (= 1), d_gate_up [R,2I].  score_partials is
  * [amoe_gated_bwd_score_parts(I, tile_cfg)][R] f32 or null; summing it over p gives the gradient
  * of row_scale[r] (amoe_score_grad_gather does that and takes the rows back to their slots).
- * bf16 only, tile_cfg 0, 1 or 2 (AMOE_ERR_UNSUPPORTED otherwise: such callers run
+ * 16-bit dtypes only, tile_cfg 0, 1 or 2 (AMOE_ERR_UNSUPPORTED otherwise: such callers run
  * amoe_grouped_gemm_nt and amoe_gated_act_bwd).  Same result as those two calls up to the rounding of d_inter to the
  * model dtype, which this path skips.
  */

@@ -129,7 +129,9 @@ def test_gated_bwd_gemm_argument_errors(lib):
     f = lib.amoe_grouped_gemm_nt_gated_bwd
     assert f(P, None, P, P, None, None, P, None, 1, 128, 4, 64, 64, 0, P, big, 0, None) == -1  # gate_up is required
     assert f(P, None, P, P, P, None, P, None, 0, 128, 4, 64, 64, 0, P, big, 0, None) == -2  # float32
-    assert b"bf16 only" in lib.amoe_last_error()
+    assert b"bf16 and float16 only" in lib.amoe_last_error()
+    assert f(P, None, P, P, P, None, P, None, 2, 128, 4, 64, 48, 0, P, big, 0, None) == -2  # float16 is accepted up to the shape checks
+    assert b"multiple of 32" in lib.amoe_last_error()
     assert f(P, None, P, P, P, None, P, None, 1, 128, 4, 64, 48, 0, P, big, 0, None) == -2  # H not a multiple of 32
     assert f(P, None, P, P, P, None, P, None, 1, 128, 4, 64, 64, 9, P, big, 0, None) == -1  # activation
     assert f(P, None, P, P, P, None, P, None, 1, 128, 4, 64, 64, 0, P, 8, 0, None) == -3  # workspace
