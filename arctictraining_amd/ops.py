@@ -298,7 +298,7 @@ def grouped_gemm_nt_gated_bwd(dy, w_down, offsets, gate_up, act: int = ACT_SILU,
                               map_ready: bool = False):
     """d_gate_up [R,2I] and score partials [n_parts,R] f32 (None unless wanted) from dy rows [.,H]
     (gathered through a_row_map), w_down [E,I,H] and the forward's gate_up [R,2I]: the data gradient
-    of the down projection with the gated-activation backward as its epilogue (bf16 only)."""
+    of the down projection with the gated-activation backward as its epilogue (bfloat16 or float16)."""
     lib = _lib.load()
     if dy.dtype not in (torch.bfloat16, torch.float16):
         raise RuntimeError("grouped_gemm_nt_gated_bwd: bfloat16 or float16 operands only")
