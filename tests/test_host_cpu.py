@@ -46,3 +46,30 @@ def test_layer_without_gate_parameter_shapes():
     gated = ArcticMoE(MoEConfig(act_fn=F.silu, input_dtype=torch.float32, intermediate_dim=6, model_dim=8,
                                 normalize_topk_scores=True, num_experts=4, top_k=2))
     assert tuple(gated.expert_gate_up.shape) == (4, 8, 12)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: --gpus above 1 exits with a message and without touching a device."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2
+    assert "ONE GPU" in r.stdout
+
+
+def test_bench_configurations_are_the_baseline_ones():
+    import importlib.util
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert set(bench.CONFIGS) == {"c1", "c2", "c3", "c4", "c5"}
+    # (dtype, T, H, E, K, I, extra): the headline configuration of the metric
+    assert bench.CONFIGS["c3"][:6] == ("bfloat16", 16384, 2048, 128, 8, 768)
+    assert bench.CONFIGS["c1"][:6] == ("float32", 2048, 512, 8, 2, 1024)
