@@ -449,10 +449,10 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
         asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "i"((ks * 16 + 4) * cpr * 16));
         return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
     };
-    auto read_a = [&](const u32x4_t* sa, auto KS, frag_t (&fa)[TM]) {
+    auto read_a = [&](const u32x4_t* sa, auto KS, frag_t (&fa)[TM], auto LIVE) {
         constexpr int ks = decltype(KS)::value;
 #pragma unroll
-        for (int t = 0; t < TM; ++t) {
+        for (int t = 0; t < decltype(LIVE)::value; ++t) {
             u32x4_t r;
             if (A_KC) {
                 const int row = wm * WTM + t * 32 + lj;
@@ -497,11 +497,12 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
     // quarter Q of a K step's MFMAs (A tile outer, B tile inner)
     constexpr int N_MFMA = TM * TN;
     static_assert(N_MFMA % 4 == 0, "a K step is issued in four chunks");
-    auto mma_quarter = [&](const frag_t (&fa)[TM], const frag_t (&fb)[TN], auto Q) {
+    auto mma_quarter = [&](const frag_t (&fa)[TM], const frag_t (&fb)[TN], auto Q, auto LIVE) {
         constexpr int q = decltype(Q)::value;
 #pragma unroll
         for (int f = q * (N_MFMA / 4); f < (q + 1) * (N_MFMA / 4); ++f) {
             const int i = f / TN, j = f % TN;
+            if (i >= decltype(LIVE)::value) continue;   // a 32-row block past the end of the expert
             acc[i][j] = Elem16<ET>::mfma(fa[i], fb[j], acc[i][j]);
         }
     };
@@ -566,54 +567,56 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
     __builtin_amdgcn_sched_barrier(0);
 
     // LOAD_B: tile kt+3 exists; LOAD_A: tile kt+4 exists; WAITN: loads younger than tile kt+1
-    auto k_tile = [&](auto LOAD_B, auto LOAD_A, auto WAITN, auto NEXT, int kt) {
+    auto k_tile = [&](auto LIVE, auto LOAD_B, auto LOAD_A, auto WAITN, auto NEXT, int kt) {
+        constexpr bool idle = decltype(LIVE)::value == 0;   // this wave owns no live row: it only takes part in the loads
         constexpr bool load_b = decltype(LOAD_B)::value, load_a = decltype(LOAD_A)::value;
         constexpr bool next = decltype(NEXT)::value;
         constexpr int waitn = decltype(WAITN)::value;
         const u32x4_t* sa = smem + (kt % NSTAGE) * STAGE;
         const u32x4_t* sb = sa + A_CH;
         // ---- step A: MFMAs on (fa0, fb0)
-        settle(fa0, fb0);
+        if (!idle) settle(fa0, fb0);
         if (B_MAP && load_b) {
             spread_b(b_snx, b_use);     // rows of the B tile whose loads go out in this step
             sfetch_b(kt + NSTAGE, b_snx);
         }
-        read_a(sa, IC1{}, fa1);
-        mma_quarter(fa0, fb0, IC0{});
+        read_a(sa, IC1{}, fa1, LIVE);
+        mma_quarter(fa0, fb0, IC0{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
-        read_b(sb, IC1{}, fb1);
-        mma_quarter(fa0, fb0, IC1{});
+        if (!idle) read_b(sb, IC1{}, fb1);
+        mma_quarter(fa0, fb0, IC1{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
         if (load_b) issue_b(kt + NSTAGE - 1, IC0{}, B_HALF{});
-        mma_quarter(fa0, fb0, IC2{});
+        mma_quarter(fa0, fb0, IC2{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
         if (load_b) issue_b(kt + NSTAGE - 1, B_HALF{}, B_ALL{});
-        mma_quarter(fa0, fb0, IC3{});
+        mma_quarter(fa0, fb0, IC3{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier<waitn>();
         __builtin_amdgcn_sched_barrier(0);
         // ---- step B: MFMAs on (fa1, fb1)
         const u32x4_t* na = smem + ((kt + 1) % NSTAGE) * STAGE;
-        settle(fa1, fb1);
+        if (!idle) settle(fa1, fb1);
         if (A_MAP && load_a) {
             spread_a(a_snx, a_use);     // rows of the A tile whose loads go out in this step
             sfetch_a(kt + NSTAGE + 1, a_snx);
         }
-        if (next) read_a(na, IC0{}, fa0);
-        mma_quarter(fa1, fb1, IC0{});
+        if (next) read_a(na, IC0{}, fa0, LIVE);
+        mma_quarter(fa1, fb1, IC0{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
-        if (next) read_b(na + A_CH, IC0{}, fb0);
-        mma_quarter(fa1, fb1, IC1{});
+        if (next && !idle) read_b(na + A_CH, IC0{}, fb0);
+        mma_quarter(fa1, fb1, IC1{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
         if (load_a) issue_a(kt + NSTAGE, IC0{}, A_HALF{});
-        mma_quarter(fa1, fb1, IC2{});
+        mma_quarter(fa1, fb1, IC2{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
         if (load_a) issue_a(kt + NSTAGE, A_HALF{}, A_ALL{});
-        mma_quarter(fa1, fb1, IC3{});
+        mma_quarter(fa1, fb1, IC3{}, LIVE);
         __builtin_amdgcn_sched_barrier(0);
     };
     // Every path through this block ends in the final k_tile, whose first action waits for the
     // fragment reads still outstanding: none is in flight when the epilogue reuses the registers.
+    auto run_tiles = [&](auto LIVE) {
     if (kt_count > 0) {
         // W<r>: loads younger than tile kt+1 when r tiles (kt included) remain and none is left to issue
         using W0 = std::integral_constant<int, 0>;
@@ -621,18 +624,43 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
         using W2 = std::integral_constant<int, 2 * PER>;
         using WFULL = std::integral_constant<int, (NSTAGE - 2) * PER>;
         static_assert(NSTAGE == 4 || NSTAGE == 5, "the drain below is written out for 4 or 5 stages");
-        read_a(smem, IC0{}, fa0);
-        read_b(smem + A_CH, IC0{}, fb0);
+        read_a(smem, IC0{}, fa0, LIVE);
+        if (decltype(LIVE)::value) read_b(smem + A_CH, IC0{}, fb0);
         __builtin_amdgcn_sched_barrier(0);
         int kt = 0;
-        for (; kt + NSTAGE < kt_count; ++kt) k_tile(T_{}, T_{}, WFULL{}, T_{}, kt);
-        if (kt + NSTAGE == kt_count) { k_tile(T_{}, F_{}, WFULL{}, T_{}, kt); ++kt; }
+        for (; kt + NSTAGE < kt_count; ++kt) k_tile(LIVE, T_{}, T_{}, WFULL{}, T_{}, kt);
+        if (kt + NSTAGE == kt_count) { k_tile(LIVE, T_{}, F_{}, WFULL{}, T_{}, kt); ++kt; }
         if (NSTAGE == 5) {
-            if (kt + 4 == kt_count) { k_tile(F_{}, F_{}, W2{}, T_{}, kt); ++kt; }
+            if (kt + 4 == kt_count) { k_tile(LIVE, F_{}, F_{}, W2{}, T_{}, kt); ++kt; }
         }
-        if (kt + 3 == kt_count) { k_tile(F_{}, F_{}, W1{}, T_{}, kt); ++kt; }
-        if (kt + 2 == kt_count) { k_tile(F_{}, F_{}, W0{}, T_{}, kt); ++kt; }
-        k_tile(F_{}, F_{}, W0{}, F_{}, kt);  // kt + 1 == kt_count here, whichever way it was reached
+        if (kt + 3 == kt_count) { k_tile(LIVE, F_{}, F_{}, W1{}, T_{}, kt); ++kt; }
+        if (kt + 2 == kt_count) { k_tile(LIVE, F_{}, F_{}, W0{}, T_{}, kt); ++kt; }
+        k_tile(LIVE, F_{}, F_{}, W0{}, F_{}, kt);  // kt + 1 == kt_count here, whichever way it was reached
+    }
+    };
+    // Only the 32-row blocks of this wave that hold live rows are read and multiplied: the last tile
+    // of an expert is often a sliver, and a block of clamped duplicate rows costs as much as a live
+    // one.  The count is wave-uniform and picks one copy of the loop; a wave without live rows still
+    // issues its share of the loads and meets the barriers.  (Tests inside one shared loop were
+    // measured slower than no skipping at all: they cost the full tiles more than the slivers gain.)
+    if constexpr (WGRAD) {
+        run_tiles(std::integral_constant<int, TM>{});
+    } else {
+        const int live_rows = min(max(mend - (m0 + wm * WTM), 0), WTM);
+        const int live = (live_rows + 31) >> 5;
+        static_assert(TM == 2 || TM == 4, "the dispatch below is written for two or four 32-row blocks per wave");
+        if (live >= TM) {
+            run_tiles(std::integral_constant<int, TM>{});
+        } else if (live == 0) {
+            run_tiles(std::integral_constant<int, 0>{});
+        } else if (live == 1) {
+            run_tiles(std::integral_constant<int, 1>{});
+        } else {
+            if constexpr (TM == 4) {
+                if (live == 2) run_tiles(std::integral_constant<int, 2>{});
+                else run_tiles(std::integral_constant<int, 3>{});
+            }
+        }
     }
 
     // ------------------------------------------------------------ epilogue

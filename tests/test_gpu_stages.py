@@ -460,6 +460,64 @@ def test_dgrad_down_with_gated_activation_backward(ops, gpu_device, cfg, act, el
                                       n_rows=R, tile_cfg=3)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("cfg", [0, 1, 3, 5])
+def test_grouped_gemm_every_sliver_height(ops, gpu_device, dtype, cfg):
+    """An expert's last tile may hold any number of live rows; a wavefront only works on its 32-row
+    blocks that hold some (one copy of the K loop per count).  Experts whose row counts leave every
+    remainder class around the block boundaries, through the plain, the transposed-weight, the fused
+    gate_up and the fused gated-backward products."""
+    _say("sliver heights", dtype, cfg)
+    g = torch.Generator().manual_seed(77)
+    rems = [1, 31, 32, 33, 63, 64, 65, 96, 97, 127, 128, 129, 160, 161, 191, 192, 193, 224, 255, 256, 0, 300]
+    counts = torch.tensor(rems)
+    E, R = len(rems), int(counts.sum())
+    cs = counts.cumsum(0)
+    offs = _offsets(counts, gpu_device)
+    H, I = 64, 160
+    d = gpu_device
+    tol = _pick(dtype, 4e-3, F32_TOL)
+    A = torch.randn(R, H, generator=g).to(dtype)
+    W = (torch.randn(E, H, 2 * I, generator=g) * 0.1).to(dtype)
+    C = ops.grouped_gemm_nn(A.to(d), W.to(d), offs, tile_cfg=cfg)
+    ref = O.grouped_gemm(A.double(), W.double(), cs)
+    assert O.rel_l2(C.cpu(), ref) <= tol, "nn"
+    # per expert as well: a wrong sliver would drown in the whole-matrix norm
+    start = 0
+    for e in range(E):
+        end = int(cs[e])
+        if end > start:
+            assert O.rel_l2(C[start:end].cpu(), ref[start:end]) <= 2 * tol, f"nn, expert {e} with {end - start} rows"
+        start = end
+    G = torch.randn(R, 2 * I, generator=g).to(dtype)
+    D = ops.grouped_gemm_nt(G.to(d), W.to(d), offs, tile_cfg=cfg)
+    refD = O.grouped_gemm(G.double(), W.double().transpose(1, 2).contiguous(), cs)
+    start = 0
+    for e in range(E):
+        end = int(cs[e])
+        if end > start:
+            assert O.rel_l2(D[start:end].cpu(), refD[start:end]) <= 2 * tol, f"nt, expert {e} with {end - start} rows"
+        start = end
+    if not (dtype == torch.float16 and cfg == 3):
+        rs = torch.rand(R, generator=g) + 0.25
+        gu, inter = ops.grouped_gemm_gateup_act_fwd(A.to(d), W.to(d), offs, 0, tile_cfg=cfg, row_scale=rs.to(d))
+        assert O.rel_l2(gu.cpu(), ref) <= tol
+        ref_inter = ref[:, 1::2] * O.activation("silu")(ref[:, 0::2]) * rs.double()[:, None]
+        assert O.rel_l2(inter.cpu(), ref_inter) <= _pick(dtype, BF16_TOL, 2e-5)
+    if cfg in (0, 1):
+        Wd = (torch.randn(E, I, H, generator=g) * 0.1).to(dtype)
+        dy = torch.randn(R, H, generator=g).to(dtype)
+        gu_in = torch.randn(R, 2 * I, generator=g).to(dtype)
+        s_perm = torch.rand(R, generator=g) + 0.1
+        d_gu, parts = ops.grouped_gemm_nt_gated_bwd(dy.to(d), Wd.to(d), offs, gu_in.to(d), 0, row_scale=s_perm.to(d), tile_cfg=cfg)
+        gu64 = gu_in.double().requires_grad_(True)
+        s64 = s_perm.double().requires_grad_(True)
+        inter64 = s64[:, None] * gu64[:, 1::2] * O.activation("silu")(gu64[:, 0::2])
+        (O.grouped_gemm(inter64, Wd.double(), cs) * dy.double()).sum().backward()
+        assert O.rel_l2(d_gu.cpu(), gu64.grad) <= _pick(dtype, 5e-3, 0.0)
+        assert O.rel_l2(parts.sum(0).cpu(), s64.grad) <= _pick(dtype, 5e-3, 0.0)
+
+
 def test_grouped_gemm_rows_outside_groups_untouched(ops, gpu_device):
     """Rows past offsets[E] are never written (the tile map covers only routed rows)."""
     g = torch.Generator().manual_seed(5)
