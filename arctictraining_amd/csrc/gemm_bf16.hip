@@ -643,10 +643,10 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
     // one.  The count is wave-uniform and picks one copy of the loop; a wave without live rows still
     // issues its share of the loads and meets the barriers.  (Tests inside one shared loop were
     // measured slower than no skipping at all: they cost the full tiles more than the slivers gain.)
-    if constexpr (WGRAD) {
-        run_tiles(std::integral_constant<int, TM>{});
-    } else {
-        const int live_rows = min(max(mend - (m0 + wm * WTM), 0), WTM);
+    {
+        // (weight gradient: mend is the number of output rows per expert; a wave whose columns all lie
+        // past the matrix edge has nothing to multiply either)
+        const int live_rows = n0 + wn * WTN < p.N ? min(max(mend - (m0 + wm * WTM), 0), WTM) : 0;
         const int live = (live_rows + 31) >> 5;
         static_assert(TM == 2 || TM == 4, "the dispatch below is written for two or four 32-row blocks per wave");
         if (live >= TM) {
