@@ -482,12 +482,12 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
     // Called before the first MFMA that consumes fragments fetched by read_tr: waits for this
     // wave's LDS reads and makes the fragments depend on the wait (an MFMA is otherwise free to
     // be scheduled ahead of it).
-    auto settle = [&](frag_t (&fa)[TM], frag_t (&fb)[TN]) {
+    auto settle = [&](frag_t (&fa)[TM], frag_t (&fb)[TN], auto LIVE) {
         if (A_KC && B_KC) return;
         asm volatile("s_waitcnt lgkmcnt(0)");
         if (!A_KC) {
 #pragma unroll
-            for (int t = 0; t < TM; ++t) asm volatile("" : "+v"(fa[t]));
+            for (int t = 0; t < decltype(LIVE)::value; ++t) asm volatile("" : "+v"(fa[t]));   // only the blocks that were read
         }
         if (!B_KC) {
 #pragma unroll
@@ -575,7 +575,7 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
         const u32x4_t* sa = smem + (kt % NSTAGE) * STAGE;
         const u32x4_t* sb = sa + A_CH;
         // ---- step A: MFMAs on (fa0, fb0)
-        if (!idle) settle(fa0, fb0);
+        if (!idle) settle(fa0, fb0, LIVE);
         if (B_MAP && load_b) {
             spread_b(b_snx, b_use);     // rows of the B tile whose loads go out in this step
             sfetch_b(kt + NSTAGE, b_snx);
@@ -596,7 +596,7 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
         __builtin_amdgcn_sched_barrier(0);
         // ---- step B: MFMAs on (fa1, fb1)
         const u32x4_t* na = smem + ((kt + 1) % NSTAGE) * STAGE;
-        if (!idle) settle(fa1, fb1);
+        if (!idle) settle(fa1, fb1, LIVE);
         if (A_MAP && load_a) {
             spread_a(a_snx, a_use);     // rows of the A tile whose loads go out in this step
             sfetch_a(kt + NSTAGE + 1, a_snx);
