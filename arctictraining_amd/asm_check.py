@@ -18,7 +18,7 @@ import subprocess
 
 _REG = re.compile(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]")
 _LABEL = re.compile(r"^(\.LBB\d+_\d+):")
-_KERNEL = re.compile(r"^(_Z\w*grouped_gemm_(?:bf16|f16)_kernel\w*):")
+_KERNEL = re.compile(r"^(_Z\w*grouped_gemm_(?:rows_)?(?:bf16|f16)_kernel\w*):")
 _BRANCH = re.compile(r"^\s*(s_cbranch_\w+|s_branch)\s+(\.LBB\d+_\d+)")
 
 
@@ -120,8 +120,36 @@ def check_kernel(lines):
 
 
 
-def check_assembly(asm_text: str, min_kernels: int = 1):
-    """Returns (number of kernels, number of transposing reads); raises RuntimeError on a violation."""
+def check_m0(lines):
+    """Every instruction that writes M0 must be followed at once (wait states aside) by the
+    direct-to-LDS load that reads it, and every such load preceded by a write: a load scheduled
+    between another load's write of M0 and that load would land in the wrong place."""
+    bad = []
+    instrs = [s for s in lines if not _LABEL.match(s)]
+    for i, s in enumerate(instrs):
+        op = s.split()[0]
+        writes_m0 = op.startswith("s_") and re.match(r"\S+\s+m0\b", s) is not None
+        if writes_m0:
+            j = i + 1
+            while j < len(instrs) and instrs[j].startswith("s_nop"):
+                j += 1
+            # (one independent vector instruction may serve as the wait state)
+            if j < len(instrs) and not instrs[j].startswith("global_load_lds") and j + 1 < len(instrs) and instrs[j][0] == "v":
+                j += 1
+            if j >= len(instrs) or not instrs[j].startswith("global_load_lds"):
+                bad.append(f"write of m0 not followed by its load: {s}")
+        if op.startswith("global_load_lds"):
+            k = i - 1
+            while k >= 0 and (instrs[k].startswith("s_nop") or instrs[k][0] == "v") and i - k <= 2:
+                k -= 1
+            if k < 0 or re.match(r"s_\S+\s+m0\b", instrs[k]) is None:
+                bad.append(f"direct-to-LDS load without a write of m0 right before it: {s}")
+    return bad
+
+
+def check_assembly(asm_text: str, min_kernels: int = 1, require_tr: bool = True):
+    """Returns (number of kernels, number of transposing reads); raises RuntimeError on a violation
+    (and, unless require_tr is False, when the text holds no transposing read at all)."""
     kernels = _kernels(asm_text.splitlines())
     if len(kernels) < min_kernels:
         raise RuntimeError(f"expected at least {min_kernels} GEMM kernels in the assembly, found {len(kernels)}")
@@ -134,10 +162,14 @@ def check_assembly(asm_text: str, min_kernels: int = 1):
         # No kernel may touch scratch (private) memory: neither spilled registers nor an index
         # array the compiler could not keep in registers (a select between freshly loaded row
         # indices once became a lookup in a scratch array and cost 5 % of the weight gradients).
+        # (only the kernels that write M0 in inline assembly: the compiler tracks its own uses)
+        m0 = check_m0(lines) if "grouped_gemm_rows_" in name else []
+        if m0:
+            raise RuntimeError(f"{name}: {m0[:3]}")
         private = [l.strip() for l in lines if re.match(r"\s*scratch_(load|store)", l)]
         if private:
             raise RuntimeError(f"{name} uses scratch memory: {private[:3]}")
-    if total_tr == 0:
+    if total_tr == 0 and require_tr:
         raise RuntimeError("no transposing reads found: the check is looking at the wrong instruction")
     return len(kernels), total_tr
 

@@ -212,3 +212,68 @@ __device__ __forceinline__ float act_bwd(float g)
         case AMOE_ACT_RELU: { constexpr int ACT = AMOE_ACT_RELU; __VA_ARGS__; } break;       \
         default: { constexpr int ACT = AMOE_ACT_GPT_OSS; __VA_ARGS__; } break;               \
     }
+
+// ---------------------------------------------------------------- tile map of the row-grouped GEMMs
+// One int4 {expert, first row, end row, 0} per bm-row tile of the expert-grouped rows, written by ONE
+// block: experts ascending, an expert's tiles in row order (its last one may be partly filled), entries
+// past the last tile hold expert -1.  An expert's short last tile stays next to its full ones on
+// purpose: the tiles of one expert share its weight panels in L2 when they are worked on together, and
+// a short tile (same loads, fewer multiplications) next to full ones evens out the memory traffic over
+// time -- a list with all the short tiles at the end was measured 4-7 % slower.
+// header[0] = number of tiles, header[1..3] = 0.
+//   row_end: inclusive scan of the experts' row counts, in LDS, visible to the block; row_base: first row of expert 0
+//   tscan [AMOE_MAX_EXPERTS]: LDS scratch
+// Called by all NTHREADS (>= 64) threads of the block.
+template <int NTHREADS>
+__device__ __forceinline__ void amoe_emit_tile_map(const int32_t* row_end, int row_base, int E, int bm, int4* tile_map,
+                                                   int32_t* header, int max_mtiles, int32_t* tscan)
+{
+    static_assert(AMOE_MAX_EXPERTS == 8 * AMOE_WAVE, "one wavefront scans 8 entries per lane");
+    const int t = threadIdx.x;
+    for (int e = t; e < AMOE_MAX_EXPERTS; e += NTHREADS) {
+        const int rows = e < E ? row_end[e] - (e ? row_end[e - 1] : 0) : 0;
+        tscan[e] = (rows + bm - 1) / bm;
+    }
+    __syncthreads();
+    if (t < AMOE_WAVE) {
+        // inclusive scan of the tile counts: 8 consecutive entries per lane, lane sums by shuffles
+        int f[8], s = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            f[i] = tscan[t * 8 + i];
+            s += f[i];
+        }
+        int inc = s;
+#pragma unroll
+        for (int o = 1; o < AMOE_WAVE; o <<= 1) {
+            const int u = __shfl_up(inc, o, AMOE_WAVE);
+            if (t >= o) inc += u;
+        }
+        int run = inc - s;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            run += f[i];
+            tscan[t * 8 + i] = run;
+        }
+    }
+    __syncthreads();
+    const int total = tscan[E - 1];
+    for (int mt = t; mt < total && mt < max_mtiles; mt += NTHREADS) {
+        // smallest ex with tscan[ex] > mt: the expert that owns tile mt
+        int lo = 0, hi = E - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (tscan[mid] > mt) hi = mid; else lo = mid + 1;
+        }
+        const int first_tile = lo ? tscan[lo - 1] : 0;
+        const int row0 = lo ? row_end[lo - 1] : 0;
+        tile_map[mt] = make_int4(lo, row_base + row0 + (mt - first_tile) * bm, row_base + row_end[lo], 0);
+    }
+    for (int mt = total + t; mt < max_mtiles; mt += NTHREADS) tile_map[mt] = make_int4(-1, 0, 0, 0);
+    if (t == 0) {
+        header[0] = total < max_mtiles ? total : max_mtiles;
+        header[1] = 0;
+        header[2] = 0;
+        header[3] = 0;
+    }
+}

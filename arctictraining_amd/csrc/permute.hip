@@ -97,57 +97,37 @@ permute_scan_kernel(int32_t* __restrict__ chunk_counts /* in: counts, out: exclu
         }
     if (t < AMOE_MAX_EXPERTS && t >= E) tot[t] = 0;
     __syncthreads();
-    // Inclusive scans over the experts of the row counts and of the per-expert tile counts, by ONE
-    // wavefront: 8 consecutive entries per lane serially, the lane sums by cross-lane shuffles
-    // (a block-wide Hillis-Steele scan costs 18 barriers of 16 wavefronts).
+    // Inclusive scan over the experts of the row counts, by ONE wavefront: 8 consecutive entries per
+    // lane serially, the lane sums by cross-lane shuffles (a block-wide Hillis-Steele scan costs 18
+    // barriers of 16 wavefronts).
     static_assert(AMOE_MAX_EXPERTS == 8 * AMOE_WAVE, "one wavefront scans 8 entries per lane");
     if (t < AMOE_WAVE) {
-        int r[8], rt[8];
-        int s_rows = 0, s_tiles = 0;
+        int r[8];
+        int s_rows = 0;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             r[i] = tot[t * 8 + i];
-            rt[i] = (r[i] + bm - 1) / bm;
             s_rows += r[i];
-            s_tiles += rt[i];
         }
-        int in_rows = s_rows, in_tiles = s_tiles;
+        int in_rows = s_rows;
 #pragma unroll
         for (int o = 1; o < AMOE_WAVE; o <<= 1) {
-            const int u = __shfl_up(in_rows, o, AMOE_WAVE), ut = __shfl_up(in_tiles, o, AMOE_WAVE);
-            if (t >= o) {
-                in_rows += u;
-                in_tiles += ut;
-            }
+            const int u = __shfl_up(in_rows, o, AMOE_WAVE);
+            if (t >= o) in_rows += u;
         }
-        int run_rows = in_rows - s_rows, run_tiles = in_tiles - s_tiles;
+        int run_rows = in_rows - s_rows;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             run_rows += r[i];
-            run_tiles += rt[i];
             tot[t * 8 + i] = run_rows;
-            tstart[t * 8 + i] = run_tiles;
         }
     }
     __syncthreads();
     if (t < E) offsets[t + 1] = tot[t];
     if (t == 0) offsets[0] = 0;
     if (tile_map == nullptr) return;
-    // tot[e] = end row of expert e, tstart[e] = first tile of expert e + 1 (inclusive scans)
-    const int total = tstart[E - 1];
-    if (t == 0) *n_mtiles = total < max_mtiles ? total : max_mtiles;
-    for (int mt = t; mt < total && mt < max_mtiles; mt += kScanThreads) {
-        // smallest ex with tstart[ex] > mt: the expert that owns tile mt
-        int lo = 0, hi = E - 1;
-        while (lo < hi) {
-            int mid = (lo + hi) >> 1;
-            if (tstart[mid] > mt) hi = mid; else lo = mid + 1;
-        }
-        const int first_tile = lo ? tstart[lo - 1] : 0;
-        const int row0 = lo ? tot[lo - 1] : 0;
-        tile_map[mt] = make_int4(lo, row0 + (mt - first_tile) * bm, tot[lo], 0);
-    }
-    for (int mt = total + t; mt < max_mtiles; mt += kScanThreads) tile_map[mt] = make_int4(-1, 0, 0, 0);
+    // tot[e] = end row of expert e
+    amoe_emit_tile_map<kScanThreads>(tot, 0, E, bm, tile_map, n_mtiles, max_mtiles, tstart);
 }
 
 __global__ void __launch_bounds__(kWavesPerBlock * AMOE_WAVE)

@@ -173,7 +173,11 @@ size_t amoe_grouped_gemm_workspace_bytes(int R, int E);
  * row_scale [R] f32 may be null (= 1); passing the row-ordered scores folds the multiply of
  * moe.py:460 into this epilogue (the down projection is linear, so scaling its input rows
  * equals scaling its output rows).  gate_up may be null when only inter is wanted.
- * tile_cfg: 0 = library default.
+ * tile_cfg: 0 = library default; 1, 2, 3, 5 = other tile shapes, for tuning.  float16 with tile_cfg 3
+ * is not built for any of the three row-grouped products (AMOE_ERR_UNSUPPORTED).
+ * A (at most R source rows of H elements) and one expert of the weights must each stay below 4 GiB:
+ * the kernels address them with 32-bit byte offsets (AMOE_ERR_UNSUPPORTED otherwise; the same holds
+ * for the two products below and for amoe_grouped_gemm_nt_gated_bwd).
  */
 int amoe_grouped_gemm_gateup_act_fwd(const void* xp, const int32_t* a_row_map, const void* w_gate_up,
                                      const int32_t* offsets, const float* row_scale, void* gate_up, void* inter,

@@ -305,9 +305,16 @@ def test_grouped_gemm_nn_nt_wgrad(ops, gpu_device, dtype, R, E, Kd, N, cname, cf
     B = (torch.randn(E, Kd, N, generator=g) * 0.1).to(dtype)
     d = gpu_device
     tol = _pick(dtype, 4e-3, F32_TOL)
+    # float16 with tile_cfg 3 exists for the weight gradient only: the row-grouped products reject it
+    rows_ok = not (dtype == torch.float16 and cfg == 3)
+    if not rows_ok:
+        with pytest.raises(RuntimeError, match="float16"):
+            ops.grouped_gemm_nn(A.to(d), B.to(d), offs, tile_cfg=cfg)
+        with pytest.raises(RuntimeError, match="float16"):
+            ops.grouped_gemm_nt(torch.randn(R, N).to(dtype).to(d), B.to(d), offs, tile_cfg=cfg)
 
     # NN: C = A @ B[e]
-    C = ops.grouped_gemm_nn(A.to(d), B.to(d), offs, tile_cfg=cfg)
+    C = ops.grouped_gemm_nn(A.to(d), B.to(d), offs, tile_cfg=cfg if rows_ok else 0)
     ref = O.grouped_gemm(A.double(), B.double(), cs)
     assert O.rel_l2(C.cpu(), ref) <= tol, "nn"
 
@@ -316,14 +323,14 @@ def test_grouped_gemm_nn_nt_wgrad(ops, gpu_device, dtype, R, E, Kd, N, cname, cf
         Tn = max(R // 2, 1)
         src = torch.randn(Tn, Kd, generator=g).to(dtype)
         rmap = torch.randint(0, Tn, (R,), generator=g)
-        C2 = ops.grouped_gemm_nn(src.to(d), B.to(d), offs, a_row_map=rmap.to(torch.int32).to(d), tile_cfg=cfg)
+        C2 = ops.grouped_gemm_nn(src.to(d), B.to(d), offs, a_row_map=rmap.to(torch.int32).to(d), tile_cfg=cfg if rows_ok else 0)
         ref2 = O.grouped_gemm(src.double()[rmap], B.double(), cs)
         assert O.rel_l2(C2.cpu(), ref2) <= tol, "nn + row map"
 
     # NT: D = G @ B[e]^T
     G = torch.randn(R, N, generator=g).to(dtype)
     if dtype == torch.float32 or (N % 32 == 0 and Kd % 8 == 0):
-        D = ops.grouped_gemm_nt(G.to(d), B.to(d), offs, tile_cfg=cfg)
+        D = ops.grouped_gemm_nt(G.to(d), B.to(d), offs, tile_cfg=cfg if rows_ok else 0)
         refD = O.grouped_gemm(G.double(), B.double().transpose(1, 2).contiguous(), cs)
         assert O.rel_l2(D.cpu(), refD) <= tol, "nt"
 
@@ -468,6 +475,8 @@ def test_grouped_gemm_every_sliver_height(ops, gpu_device, dtype, cfg):
     remainder class around the block boundaries, through the plain, the transposed-weight, the fused
     gate_up and the fused gated-backward products."""
     _say("sliver heights", dtype, cfg)
+    if dtype == torch.float16 and cfg == 3:
+        pytest.skip("float16 with tile_cfg 3 exists for the weight gradient only")
     g = torch.Generator().manual_seed(77)
     rems = [1, 31, 32, 33, 63, 64, 65, 96, 97, 127, 128, 129, 160, 161, 191, 192, 193, 224, 255, 256, 0, 300]
     counts = torch.tensor(rems)

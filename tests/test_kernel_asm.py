@@ -27,7 +27,9 @@ def test_transposing_reads_are_awaited_before_use(tmp_path):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         pytest.skip("hipcc not available")
-    flags = [f for f in HIPCC_FLAGS if f not in ("-fPIC", "-fvisibility=hidden")]
+    # one of the four groups the build compiles (the plain row-grouped products: persistent kernel,
+    # K-strided B operand read with the transposing read); the build itself checks all four
+    flags = [f for f in HIPCC_FLAGS if f not in ("-fPIC", "-fvisibility=hidden")] + ["-DAMOE_GEMM_PART=1"]
     asm = asm_check.compile_to_assembly(os.path.join(SRC_DIR, "gemm_bf16.hip"), str(tmp_path / "gemm_bf16.s"), flags)
-    n_kernels, n_tr = asm_check.check_assembly(asm, min_kernels=20)
-    assert n_kernels >= 20 and n_tr > 0
+    n_kernels, n_tr = asm_check.check_assembly(asm, min_kernels=10)
+    assert n_kernels >= 10 and n_tr > 0
