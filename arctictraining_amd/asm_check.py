@@ -18,7 +18,7 @@ import subprocess
 
 _REG = re.compile(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]")
 _LABEL = re.compile(r"^(\.LBB\d+_\d+):")
-_KERNEL = re.compile(r"^(_Z\w*grouped_gemm_(?:rows_)?(?:bf16|f16)_kernel\w*):")
+_KERNEL = re.compile(r"^(_Z\w*grouped_gemm_(?:rows|wgrad)_(?:bf16|f16)_kernel\w*):")
 _BRANCH = re.compile(r"^\s*(s_cbranch_\w+|s_branch)\s+(\.LBB\d+_\d+)")
 
 

@@ -1,9 +1,11 @@
-// Ragged grouped GEMMs on bf16 MFMA (v_mfma_f32_32x32x16_bf16), f32 accumulate.
+// Ragged grouped GEMMs on bf16 / f16 MFMA (v_mfma_f32_32x32x16_bf16 / _f16), f32 accumulate.
 //
-// One kernel template covers the three operand layouts of the expert FFN:
-//   rows / NN   C[rows_e,:] = A[rows_e,:] @ B[e]        (forward; B is [Kd,N], N contiguous)
-//   rows / NT   C[rows_e,:] = A[rows_e,:] @ B[e]^T      (data gradient; B is [N',Kd'] so both K-contiguous)
-//   wgrad / TN  C[e] = A[rows_e,:]^T @ B[rows_e,:]      (weight gradient; the reduction runs over the ragged rows)
+// Two kernel templates cover the three operand layouts of the expert FFN:
+//   grouped_gemm_rows_body (persistent, one workgroup per CU)
+//     rows / NN   C[rows_e,:] = A[rows_e,:] @ B[e]        (forward; B is [Kd,N], N contiguous)
+//     rows / NT   C[rows_e,:] = A[rows_e,:] @ B[e]^T      (data gradient; B is [N',Kd'] so both K-contiguous)
+//   grouped_gemm_wgrad_body (one tile per workgroup)
+//     wgrad / TN  C[e] = A[rows_e,:]^T @ B[rows_e,:]      (weight gradient; the reduction runs over the ragged rows)
 //
 // Tiles of BM x BN x 32 move from global memory straight into LDS (global_load_lds, 16 bytes
 // per lane, four stages in flight); the XOR swizzle of the LDS layout is applied on the source
@@ -25,8 +27,8 @@
 //
 // Row-grouped launches take their (expert, first row, end row) per M tile from a tile map
 // that a small kernel builds on the device from the expert offsets: no host sync, empty
-// experts simply own no tile.  Workgroups are dealt to the 8 XCDs so that the ~32 resident on
-// one XCD cover one super-tile of gm x gn tiles (shared A and B panels in that XCD's L2),
+// experts simply own no tile.  Tiles are dealt to the 8 XCDs so that the ~32 workgroups resident
+// on one XCD cover one super-tile of gm x gn tiles (shared A and B panels in that XCD's L2),
 // and super-tiles rotate over the XCDs, which keeps them evenly loaded whatever the routing
 // skew.
 #include "amoe_common.h"
@@ -228,19 +230,19 @@ __device__ __forceinline__ void act_both_fast(float g, float& f, float& df)
 using T_ = std::true_type;
 using F_ = std::false_type;
 
-// MAPS (weight gradient only): 1 = the rows of A, 2 = the rows of B are gathered through a row map
+// ------------------------------------------------------------------ weight gradient: one tile per workgroup
+// C[e] = A[rows_e,:]^T @ B[rows_e,:]: the reduction runs over the expert's rows, both operands are
+// K-strided ([k][column] in LDS, transposing reads).
+// MAPS: 1 = the rows of A, 2 = the rows of B are gathered through a row map
 // ET: the 16-bit element type (bf16_t or f16_t); GemmArgs names its pointers bf16_t for both
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS, typename ET>
-__device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
+template <int BM, int BN, int WGM, int WGN, int MAPS, typename ET>
+__device__ __forceinline__ void grouped_gemm_wgrad_body(const GemmArgs& p)
 {
     typedef typename Elem16<ET>::frag_t frag_t;
     constexpr int NT = WGM * WGN * 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr bool WGRAD = !A_KC;
-    constexpr bool A_MAP = WGRAD && (MAPS & 1), B_MAP = WGRAD && (MAPS & 2);
-    static_assert(WGRAD || MAPS == 0, "row-grouped launches gather through the per-thread row plan");
-    static_assert(!WGRAD || !B_KC, "the weight gradient reduces over rows: both operands are K-strided");
+    constexpr bool A_MAP = (MAPS & 1) != 0, B_MAP = (MAPS & 2) != 0;
     static_assert(BM >= 128 && BN >= 128, "K-strided swizzle needs 16 chunks per row");
     constexpr int A_CH = BM * 4, B_CH = BN * 4;   // 16-byte chunks per stage (a 32-wide K row is 4 chunks)
     constexpr int STAGE = A_CH + B_CH;
@@ -269,28 +271,12 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
     const int pm = sm * p.gm + w / p.gn;
     const int nt = sn_i * p.gn + w % p.gn;
     if (nt >= p.n_ntiles) return;
-    int e, m0, mend, kt_count;
-    int r0 = 0, r1 = 0;
-    if (!WGRAD) {
-        if (pm >= p.max_mtiles) return;
-        int4 tm = p.tile_map[pm];
-        // the whole entry in one load (pinned here; otherwise .y and .z are fetched by a second,
-        // dependent load behind the test of .x)
-        asm volatile("" : "+s"(tm.x), "+s"(tm.y), "+s"(tm.z));
-        if (tm.x < 0) return;
-        e = tm.x;
-        m0 = tm.y;
-        mend = tm.z;
-        kt_count = p.Kd / BK;
-    } else {
-        e = pm / p.n_mt;
-        if (e >= p.E) return;
-        m0 = (pm - e * p.n_mt) * BM;
-        mend = p.M;
-        r0 = p.offsets[e];
-        r1 = p.offsets[e + 1];
-        kt_count = (r1 - r0 + BK - 1) / BK;
-    }
+    const int e = pm / p.n_mt;
+    if (e >= p.E) return;
+    const int m0 = (pm - e * p.n_mt) * BM;
+    const int mend = p.M;   // output rows per expert
+    const int r0 = p.offsets[e], r1 = p.offsets[e + 1];
+    const int kt_count = (r1 - r0 + BK - 1) / BK;
     const int n0 = nt * BN;
 
     // ------------------------------------------------------------ global load plans
@@ -302,52 +288,27 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
     int a_kr[PER_A], b_kr[PER_B];  // wgrad: k row of the chunk, for the ragged-end mask
     const bf16_t* Ab = p.A;
     const bf16_t* Bb = p.B;
-    // Gated epilogue: thread r < BM fetches the scale of tile row r now and parks it in LDS once
-    // the main loop has released the stages.  Loading the scales in the epilogue would put
-    // vector loads between the stores, and a load result can only be awaited together with every
-    // store issued before it.
-    float rs_in = 1.0f;
-    if (EPI != EPI_STORE && tid < BM && p.row_scale) rs_in = p.row_scale[min(m0 + tid, mend - 1)];
 #pragma unroll
     for (int i = 0; i < PER_A; ++i) {
         const int c = tid + NT * i;
-        if (A_KC) {
-            const int row = c >> 2, kc = (c & 3) ^ ((row >> 2) & 3);
-            int gr = min(m0 + row, mend - 1);
-            if (p.a_row_map) gr = p.a_row_map[gr];
-            aoff[i] = (uint32_t)gr * (uint32_t)p.lda + kc * 8;
-            a_kr[i] = 0;
-        } else {
-            constexpr int CPR = BM / 8;
-            const int krow = c / CPR, mc = (c % CPR) ^ ((krow & 3) << 2);
-            const int col = min(m0 + mc * 8, p.M - 8);
-            aoff[i] = A_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.lda + col;
-            a_kr[i] = krow;
-        }
+        constexpr int CPR = BM / 8;
+        const int krow = c / CPR, mc = (c % CPR) ^ ((krow & 3) << 2);
+        const int col = min(m0 + mc * 8, p.M - 8);
+        aoff[i] = A_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.lda + col;
+        a_kr[i] = krow;
     }
 #pragma unroll
     for (int i = 0; i < PER_B; ++i) {
         const int c = tid + NT * i;
-        if (B_KC) {
-            const int row = c >> 2, kc = (c & 3) ^ ((row >> 2) & 3);
-            const int gn = min(n0 + row, p.N - 1);
-            boff[i] = (uint32_t)gn * (uint32_t)p.ldb + kc * 8;
-            b_kr[i] = 0;
-        } else {
-            constexpr int CPR = BN / 8;
-            const int krow = c / CPR, nc = (c % CPR) ^ ((krow & 3) << 2);
-            const int col = min(n0 + nc * 8, p.N - 8);
-            boff[i] = B_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.ldb + col;
-            b_kr[i] = krow;
-        }
+        constexpr int CPR = BN / 8;
+        const int krow = c / CPR, nc = (c % CPR) ^ ((krow & 3) << 2);
+        const int col = min(n0 + nc * 8, p.N - 8);
+        boff[i] = B_MAP ? (uint32_t)col : (uint32_t)krow * (uint32_t)p.ldb + col;
+        b_kr[i] = krow;
     }
-    if (!WGRAD) {
-        Bb += (long long)e * p.strideB;
-    } else {
-        if (!A_MAP) Ab += (long long)r0 * p.lda;
-        if (!B_MAP) Bb += (long long)r0 * p.ldb;
-    }
-    const int k_rows = r1 - r0;  // wgrad: rows of this expert
+    if (!A_MAP) Ab += (long long)r0 * p.lda;
+    if (!B_MAP) Bb += (long long)r0 * p.ldb;
+    const int k_rows = r1 - r0;  // rows of this expert
 
     // Gathered operands of the weight gradient: the source row of a chunk changes with every K
     // tile.  One wave-wide load covers RPW consecutive k rows starting at a wave-uniform row, so
@@ -411,12 +372,12 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
         constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
         const int k0 = kt * BK;
         u32x4_t* sa = smem + (kt % NSTAGE) * STAGE + wave * 64;
-        const bf16_t* a_base = A_KC ? Ab + k0 : (A_MAP ? Ab : Ab + (long long)k0 * p.lda);
+        const bf16_t* a_base = A_MAP ? Ab : Ab + (long long)k0 * p.lda;
 #pragma unroll
         for (int i = lo; i < hi; ++i) {
             const bf16_t* src = a_base + aoff[i];
             if (A_MAP) src += (long long)idx[i] * p.lda;
-            if (WGRAD) src = (k0 + a_kr[i] < k_rows) ? src : zero_src;
+            src = (k0 + a_kr[i] < k_rows) ? src : zero_src;
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sa + NT * i), 16, 0, 0);
         }
     };
@@ -424,12 +385,12 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
         constexpr int lo = decltype(LO)::value, hi = decltype(HI)::value;
         const int k0 = kt * BK;
         u32x4_t* sb = smem + (kt % NSTAGE) * STAGE + A_CH + wave * 64;
-        const bf16_t* b_base = B_KC ? Bb + k0 : (B_MAP ? Bb : Bb + (long long)k0 * p.ldb);
+        const bf16_t* b_base = B_MAP ? Bb : Bb + (long long)k0 * p.ldb;
 #pragma unroll
         for (int i = lo; i < hi; ++i) {
             const bf16_t* src = b_base + boff[i];
             if (B_MAP) src += (long long)idx[i] * p.ldb;
-            if (WGRAD) src = (k0 + b_kr[i] < k_rows) ? src : zero_src;
+            src = (k0 + b_kr[i] < k_rows) ? src : zero_src;
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(sb + NT * i), 16, 0, 0);
         }
     };
@@ -445,8 +406,7 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     // ------------------------------------------------------------ fragment readers
-    // One 16-byte register quad per 32-wide tile and 16-deep K step, whatever the layout.
-    // K-strided operands: lane -> (k row, 4 columns) inside the 4x16 block its 16-lane group
+    // One 16-byte register quad per 32-wide tile and 16-deep K step.  Lane -> (k row, 4 columns) inside the 4x16 block its 16-lane group
     // transposes; groups 0/1 take columns 0-15 / 16-31 of the tile, groups 2/3 the k rows 8-15.
     // The transposing read is issued as inline assembly: through the builtin the compiler treats
     // it as possibly aliasing the direct-to-LDS loads in flight and drains them all (vmcnt(0))
@@ -469,46 +429,25 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
         constexpr int ks = decltype(KS)::value;
 #pragma unroll
         for (int t = 0; t < decltype(LIVE)::value; ++t) {
-            u32x4_t r;
-            if (A_KC) {
-                const int row = wm * WTM + t * 32 + lj;
-                const int kc = ks * 2 + lg;
-                r = sa[row * 4 + (kc ^ ((row >> 2) & 3))];
-            } else {
-                r = read_tr(sa, std::integral_constant<int, BM / 8>{}, wm * WTM + t * 32, KS);
-            }
-            fa[t] = __builtin_bit_cast(frag_t, r);
+            fa[t] = __builtin_bit_cast(frag_t, read_tr(sa, std::integral_constant<int, BM / 8>{}, wm * WTM + t * 32, KS));
         }
     };
     auto read_b = [&](const u32x4_t* sb, auto KS, frag_t (&fb)[TN]) {
         constexpr int ks = decltype(KS)::value;
 #pragma unroll
         for (int t = 0; t < TN; ++t) {
-            u32x4_t r;
-            if (B_KC) {
-                const int row = wn * WTN + t * 32 + lj;
-                const int kc = ks * 2 + lg;
-                r = sb[row * 4 + (kc ^ ((row >> 2) & 3))];
-            } else {
-                r = read_tr(sb, std::integral_constant<int, BN / 8>{}, wn * WTN + t * 32, KS);
-            }
-            fb[t] = __builtin_bit_cast(frag_t, r);
+            fb[t] = __builtin_bit_cast(frag_t, read_tr(sb, std::integral_constant<int, BN / 8>{}, wn * WTN + t * 32, KS));
         }
     };
     // Called before the first MFMA that consumes fragments fetched by read_tr: waits for this
     // wave's LDS reads and makes the fragments depend on the wait (an MFMA is otherwise free to
     // be scheduled ahead of it).
     auto settle = [&](frag_t (&fa)[TM], frag_t (&fb)[TN], auto LIVE) {
-        if (A_KC && B_KC) return;
         asm volatile("s_waitcnt lgkmcnt(0)");
-        if (!A_KC) {
 #pragma unroll
-            for (int t = 0; t < decltype(LIVE)::value; ++t) asm volatile("" : "+v"(fa[t]));   // only the blocks that were read
-        }
-        if (!B_KC) {
+        for (int t = 0; t < decltype(LIVE)::value; ++t) asm volatile("" : "+v"(fa[t]));   // only the blocks that were read
 #pragma unroll
-            for (int t = 0; t < TN; ++t) asm volatile("" : "+v"(fb[t]));
-        }
+        for (int t = 0; t < TN; ++t) asm volatile("" : "+v"(fb[t]));
     };
     // quarter Q of a K step's MFMAs (A tile outer, B tile inner)
     constexpr int N_MFMA = TM * TN;
@@ -681,44 +620,22 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
 
     // ------------------------------------------------------------ epilogue
     // Lane l of tile (i, j) holds column j*32 + l%32 for 16 rows; registers v, v+1 (v even) are
-    // rows r, r+1.  Each lane converts its two values to one packed bf16 pair, lanes 2c and 2c+1
+    // rows r, r+1.  Each lane converts its two values to one packed pair, lanes 2c and 2c+1
     // exchange the pairs (DPP) and a byte permute leaves the even lane with columns (2c, 2c+1) of
     // row r and the odd lane with those of row r+1: three VALU operations per 4-byte store.
-    // Gated: that pair is (gate, up) of intermediate column c; a second exchange between lanes l
-    // and l^2 over two row pairs packs two neighbouring intermediate columns of one row.
     // Addresses are a wave-uniform row base (scalar arithmetic) plus one per-lane 32-bit offset;
-    // tiles that lie entirely inside their expert's rows and the matrix take the FULL form
-    // without per-store bounds tests.
-    bf16_t* Cb = WGRAD ? p.C + (long long)e * p.strideC : p.C;
-    const int odd1 = lj & 1, odd2 = (lj >> 1) & 1;
-    float* s_rs = reinterpret_cast<float*>(smem);   // the stages are free once every wave is past the loop
-    if (EPI != EPI_STORE) {
-        __syncthreads();
-        if (tid < BM) s_rs[tid] = rs_in;
-        __syncthreads();
-    }
+    // tiles that lie entirely inside the matrix take the FULL form without per-store bounds tests.
+    bf16_t* Cb = p.C + (long long)e * p.strideC;
+    const int odd1 = lj & 1;
     const uint32_t swap_sel = odd1 ? 0x03020706u : 0x05040100u;
     // wave-uniform origin of this wave's part of the tile, and the lane's offset from it (bytes)
     const long long worg = (long long)(m0 + wm * WTM) * p.ldc + n0 + wn * WTN;
-    const long long worg2 = (long long)(m0 + wm * WTM) * p.ldc2 + ((n0 + wn * WTN) >> 1);
-    char* cbase = reinterpret_cast<char*>((EPI == EPI_GATED ? p.C : Cb) + worg);
-    char* c2base = EPI == EPI_GATED ? reinterpret_cast<char*>(p.C2 + worg2) : nullptr;
+    char* cbase = reinterpret_cast<char*>(Cb + worg);
     const uint32_t loff = (uint32_t)((4 * lg + odd1) * p.ldc + (lj & ~1)) * 2u;
-    const uint32_t loff2 = EPI == EPI_GATED ? (uint32_t)((4 * lg + 2 * odd2 + odd1) * p.ldc2 + ((lj >> 1) & ~1)) * 2u : 0u;
-    const bool want_c = EPI != EPI_GATED || p.C != nullptr;
     auto epilogue = [&](auto FULL) {
         constexpr bool full = decltype(FULL)::value;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            // gated: the scales of this lane's 8 rows of tile row i, fetched together ahead of
-            // the column loop (one wait for the batch instead of one per use)
-            float sc[4][2];
-            if (EPI == EPI_GATED) {
-#pragma unroll
-                for (int v4 = 0; v4 < 4; ++v4)
-#pragma unroll
-                    for (int u = 0; u < 2; ++u) sc[v4][u] = s_rs[wm * WTM + i * 32 + 8 * v4 + 4 * lg + 2 * u + odd1];
-            }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const bool col_ok = full || (n0 + wn * WTN + j * 32 + (lj & ~1) < p.N);
@@ -726,131 +643,21 @@ __device__ __forceinline__ void grouped_gemm_body(const GemmArgs& p)
                 for (int v = 0; v < 16; v += 4) {
                     const int rq = i * 32 + 8 * (v >> 2);           // first of 8 rows, relative to the wave's origin
                     const int rt = wm * WTM + rq + 4 * lg;          // rows rt..rt+3 of the tile
-                    float h[2];
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
                         const uint32_t own = Elem16<ET>::pack2(acc[i][j][v + 2 * u], acc[i][j][v + 2 * u + 1]);
                         const uint32_t got = __builtin_amdgcn_update_dpp(0, own, 0xB1, 0xF, 0xF, true);
                         const uint32_t pk = __builtin_amdgcn_perm(got, own, swap_sel);
                         const bool ok = full || (col_ok && m0 + rt + 2 * u + odd1 < mend);
-                        if (EPI == EPI_GATED)
-                            h[u] = sc[v >> 2][u] * Elem16<ET>::hi(pk) * act_fwd_fast<ACT>(Elem16<ET>::lo(pk));
-                        if (want_c && ok) {
+                        if (ok) {
                             char* rowp = cbase + ((long long)(rq + 2 * u) * p.ldc + j * 32) * 2;
                             *reinterpret_cast<uint32_t*>(rowp + loff) = pk;
-                        }
-                    }
-                    if (EPI == EPI_GATED) {
-                        // lanes with bit 1 clear keep the first row pair, the others the second
-                        const float got = lane_xor2(odd2 ? h[0] : h[1]);
-                        const uint32_t hp = odd2 ? Elem16<ET>::pack2(got, h[1]) : Elem16<ET>::pack2(h[0], got);
-                        const bool ok = full || (col_ok && m0 + rt + 2 * odd2 + odd1 < mend);
-                        if (ok) {
-                            char* rowp = c2base + ((long long)rq * p.ldc2 + j * 16) * 2;
-                            *reinterpret_cast<uint32_t*>(rowp + loff2) = hp;
                         }
                     }
                 }
             }
         }
     };
-    if (EPI == EPI_GATED_BWD) {
-        // The accumulators are d_inter[r, c] (c = intermediate column); nothing of it is stored.
-        // With (gate, up) = gate_up[r, 2c], gate_up[r, 2c+1] re-read from the forward pass and
-        // s = row_scale[r]:  d_gate_up[r, 2c] = s * d * up * act'(gate),  d_gate_up[r, 2c+1] =
-        // s * d * act(gate)  (one packed pair per element, no lane exchange needed), and the row
-        // sums  sum_c d * up * act(gate)  -- the gradient of s -- are reduced over the tile's columns
-        // in a fixed order and written to partials[N tile][row].
-        float* s_part = s_rs + BM;   // [2 * WGN][BM] partial row sums of the half-wave column groups
-        // gate_up and d_gate_up have the same [R, 2N] shape: one wave-uniform origin each (scalar
-        // arithmetic per element row) plus one per-lane byte offset shared by both
-        const long long gorg = (long long)(m0 + wm * WTM) * p.ldg + 2 * (n0 + wn * WTN);
-        const char* gbase = reinterpret_cast<const char*>(p.G + gorg);
-        char* dbase = reinterpret_cast<char*>(p.C + gorg);
-        const uint32_t goff = (uint32_t)(4 * lg * p.ldg + 2 * lj) * 2u;
-        auto run = [&](auto FULL) {
-            constexpr bool full = decltype(FULL)::value;
-            // a block = 8 of the 16 values a lane holds of one 32x32 tile (half hh: registers 8hh..8hh+7)
-            auto load_block = [&](int i, int j, int hh, uint32_t (&g)[8]) {
-                const bool col_ok = full || (n0 + wn * WTN + j * 32 + lj < p.N);
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int v = 8 * hh + u;
-                    const int rr = i * 32 + 8 * (v >> 2) + (v & 3);   // row relative to the wave's origin (+ 4*lg in goff)
-                    const bool ok = full || (col_ok && m0 + wm * WTM + rr + 4 * lg < mend);
-                    const char* rowp = gbase + ((long long)rr * p.ldg + 2 * j * 32) * 2;
-                    g[u] = ok ? *reinterpret_cast<const uint32_t*>(rowp + goff) : 0u;
-                }
-            };
-            uint32_t gcur[8], gnxt[8];
-            load_block(0, 0, 0, gcur);
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                float dot[16];
-#pragma unroll
-                for (int v = 0; v < 16; ++v) dot[v] = 0.f;
-#pragma unroll
-                for (int jh = 0; jh < 2 * TN; ++jh) {
-                    const int j = jh >> 1, hh = jh & 1;
-                    // the next block's pairs are requested before this block is worked on
-                    constexpr int NB = TM * TN * 2;
-                    const int b_next = i * 2 * TN + jh + 1;
-                    if (b_next < NB) load_block(b_next / (2 * TN), (b_next % (2 * TN)) >> 1, b_next & 1, gnxt);
-                    __builtin_amdgcn_sched_barrier(0);
-                    const bool col_ok = full || (n0 + wn * WTN + j * 32 + lj < p.N);
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        // (fenced every four elements: left alone, the scheduler interleaves all the
-                        // activation chains and their temporaries no longer fit beside the accumulators)
-                        if (u == 4) __builtin_amdgcn_sched_barrier(0);
-                        const int v = 8 * hh + u;
-                        const int rr = i * 32 + 8 * (v >> 2) + (v & 3);
-                        const float d = acc[i][j][v];
-                        const float gate = Elem16<ET>::lo(gcur[u]), up = Elem16<ET>::hi(gcur[u]);
-                        float f, df;
-                        act_both_fast<ACT>(gate, f, df);
-                        const float sd = s_rs[wm * WTM + rr + 4 * lg] * d;
-                        dot[v] += d * up * f;
-                        const bool ok = full || (col_ok && m0 + wm * WTM + rr + 4 * lg < mend);
-                        if (ok) {
-                            char* rowp = dbase + ((long long)rr * p.ldg + 2 * j * 32) * 2;
-                            *reinterpret_cast<uint32_t*>(rowp + goff) = Elem16<ET>::pack2(sd * up * df, sd * f);
-                        }
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (b_next < NB) {
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) gcur[u] = gnxt[u];
-                    }
-                }
-                if (p.partials) {
-                    // sum over the 16 lanes of a row group (its 16 columns), then one slot per
-                    // (wave column, half-wave group) and tile row
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        float x = dot[v];
-                        x += dpp_f32<AMOE_DPP_QUAD_XOR1>(x);
-                        x += dpp_f32<AMOE_DPP_QUAD_XOR2>(x);
-                        x += dpp_f32<AMOE_DPP_HALF_MIRROR>(x);
-                        x += dpp_f32<AMOE_DPP_MIRROR>(x);
-                        if ((lane & 15) == 0)
-                            s_part[(wn * 2 + ((lane >> 4) & 1)) * BM + wm * WTM + i * 32 + 8 * (v >> 2) + 4 * lg + (v & 3)] = x;
-                    }
-                }
-            }
-        };
-        if (m0 + BM <= mend && n0 + BN <= p.N) run(T_{}); else run(F_{});
-        if (p.partials) {
-            __syncthreads();
-            if (tid < BM && m0 + tid < mend) {
-                float tot = 0.f;
-#pragma unroll
-                for (int q = 0; q < 2 * WGN; ++q) tot += s_part[q * BM + tid];
-                p.partials[(long long)nt * p.part_stride + m0 + tid] = tot;
-            }
-        }
-        return;
-    }
     if (m0 + BM <= mend && n0 + BN <= p.N) epilogue(T_{}); else epilogue(F_{});
 }
 
@@ -981,7 +788,7 @@ __device__ __forceinline__ void grouped_gemm_rows_body(const GemmArgs& p)
 
     mfma_f32x16 acc[TM][TN];
 
-    // ------------------------------------------------------------ fragment readers (see grouped_gemm_body)
+    // ------------------------------------------------------------ fragment readers (see grouped_gemm_wgrad_body)
     const int tr_j = lane & 15, tr_blk = lane >> 4;
     const int tr_col = 16 * (tr_blk & 1) + 4 * (tr_j & 3);
     const int tr_k = 8 * (tr_blk >> 1) + (tr_j >> 2);
@@ -1445,19 +1252,19 @@ __device__ __forceinline__ void grouped_gemm_rows_body(const GemmArgs& p)
 
 // ------------------------------------------------------------------ host side
 
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
+template <int BM, int BN, int WGM, int WGN, int MAPS>
 __global__ void __launch_bounds__(WGM * WGN * 64)
-grouped_gemm_bf16_kernel(GemmArgs p)
+grouped_gemm_wgrad_bf16_kernel(GemmArgs p)
 {
-    grouped_gemm_body<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS, bf16_t>(p);
+    grouped_gemm_wgrad_body<BM, BN, WGM, WGN, MAPS, bf16_t>(p);
 }
 
 // the same kernel on float16 operands (v_mfma_f32_32x32x16_f16)
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, int EPI, int ACT, int MAPS = 0>
+template <int BM, int BN, int WGM, int WGN, int MAPS>
 __global__ void __launch_bounds__(WGM * WGN * 64)
-grouped_gemm_f16_kernel(GemmArgs p)
+grouped_gemm_wgrad_f16_kernel(GemmArgs p)
 {
-    grouped_gemm_body<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS, f16_t>(p);
+    grouped_gemm_wgrad_body<BM, BN, WGM, WGN, MAPS, f16_t>(p);
 }
 
 template <int BM, int BN, int WGM, int WGN, bool B_KC, int EPI, int ACT>
@@ -1533,9 +1340,9 @@ int launch_cfg(const GemmArgs& a, int grid, hipStream_t s)
         return launch_kernel<grouped_gemm_rows_bf16_kernel<BM, BN, WGM, WGN, B_KC, EPI, ACT>, NT, lds_bytes>(a, g, s);
     } else {
         if constexpr (F16_OK) {
-            if (a.f16) return launch_kernel<grouped_gemm_f16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS>, NT, stage_bytes>(a, grid, s);
+            if (a.f16) return launch_kernel<grouped_gemm_wgrad_f16_kernel<BM, BN, WGM, WGN, MAPS>, NT, stage_bytes>(a, grid, s);
         }
-        return launch_kernel<grouped_gemm_bf16_kernel<BM, BN, WGM, WGN, A_KC, B_KC, EPI, ACT, MAPS>, NT, stage_bytes>(a, grid, s);
+        return launch_kernel<grouped_gemm_wgrad_bf16_kernel<BM, BN, WGM, WGN, MAPS>, NT, stage_bytes>(a, grid, s);
     }
 }
 

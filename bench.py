@@ -287,13 +287,15 @@ def main():
     tile = {1: "128, 128, 2, 2", 2: "256, 128, 2, 2", 3: "256, 256, 2, 2", 5: "256, 256, 4, 2"}.get(c, "256, 256, 2, 4")
     gathered = token_of is not None
     sym = {
-        "gemm_gateup_act_fwd": f"grouped_gemm_bf16_kernel<{tile}, true, false, 1, 0, 0>",
-        "gemm_down_fwd": f"grouped_gemm_bf16_kernel<{tile}, true, false, 0, 0, 0>",
-        "gemm_dgrad_down": f"grouped_gemm_bf16_kernel<{tile}, true, true, 0, 0, 0>",
-        "gemm_dgrad_down_gated_bwd": f"grouped_gemm_bf16_kernel<{tile}, true, true, 2, 0, 0>",
-        "gemm_dgrad_gateup": f"grouped_gemm_bf16_kernel<{tile}, true, true, 0, 0, 0>",
-        "gemm_wgrad_down": f"grouped_gemm_bf16_kernel<{tile}, false, false, 0, 0, {2 if gathered else 0}>",
-        "gemm_wgrad_gateup": f"grouped_gemm_bf16_kernel<{tile}, false, false, 0, 0, {1 if gathered else 0}>",
+        # grouped_gemm_rows_bf16_kernel<BM, BN, waves along M, waves along N, B K-contiguous, epilogue, activation>
+        "gemm_gateup_act_fwd": f"grouped_gemm_rows_bf16_kernel<{tile}, false, 1, 0>",
+        "gemm_down_fwd": f"grouped_gemm_rows_bf16_kernel<{tile}, false, 0, 0>",
+        "gemm_dgrad_down": f"grouped_gemm_rows_bf16_kernel<{tile}, true, 0, 0>",
+        "gemm_dgrad_down_gated_bwd": f"grouped_gemm_rows_bf16_kernel<{tile}, true, 2, 0>",
+        "gemm_dgrad_gateup": f"grouped_gemm_rows_bf16_kernel<{tile}, true, 0, 0>",
+        # grouped_gemm_wgrad_bf16_kernel<BM, BN, waves along M, waves along N, gathered operand>
+        "gemm_wgrad_down": f"grouped_gemm_wgrad_bf16_kernel<{tile}, {2 if gathered else 0}>",
+        "gemm_wgrad_gateup": f"grouped_gemm_wgrad_bf16_kernel<{tile}, {1 if gathered else 0}>",
     }
     if dtype != torch.bfloat16:
         sym = {k: "grouped_gemm_f32_kernel" for k in sym}
