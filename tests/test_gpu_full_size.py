@@ -10,6 +10,8 @@ checked through what does not grow with the size:
     formulas of the backward: dW_down[e][i,:] = sum_r inter_s[r,i] dy[tok_r,:], dW_gate_up[e][:,c]
     = sum_r x[tok_r,:] d_gate_up[r,c]) evaluated in float64 over exactly the rows of that expert.
 C4 has no router: its grouped GEMMs are checked on sampled rows and elements the same way.
+C3 and C5 are additionally checked in FULL (test_full_size_every_row_and_expert): every row of y and
+dx, every expert of both weight gradients, against the reference's formulas in float32 on the device.
 """
 import numpy as np
 import pytest
@@ -198,6 +200,121 @@ def test_full_size_router_gradient(gpu_device, name):
     assert err <= TOL
 
 
+def _device_reference(x, wr, wgu, wd, dy, cap, K):
+    """The default path of the reference (moe.py:54-60 grouped product as a per-expert matmul loop,
+    :176-193 gated FFN, :340-357 gather, :450-461 combine) and the stage formulas of its backward, in
+    float32 torch ops on the device, over the routing the layer captured (the routing itself is
+    compared bit for bit elsewhere).  Intermediates the reference stores in the model dtype are
+    rounded to it.  Returns y, the expert part of dx, both weight gradients and the score gradients."""
+    bf = torch.bfloat16
+    T, H = x.shape
+    E, _, I2 = wgu.shape
+    tok = cap["token_of"].long()
+    offs = cap["offsets"].cpu().tolist()
+    s_perm = cap["scores"].t().reshape(-1)[cap["slot_of"].long()].float()     # k-major flatten, row order
+    xp = x[tok].float()
+    R = tok.numel()
+    gate_up = torch.empty(R, I2, device=x.device, dtype=bf)
+    for e in range(E):
+        if offs[e + 1] > offs[e]:
+            gate_up[offs[e]:offs[e + 1]] = (xp[offs[e]:offs[e + 1]] @ wgu[e].float()).to(bf)
+    gate, up = gate_up[:, 0::2].float(), gate_up[:, 1::2].float()
+    inter = (up * F.silu(gate)).to(bf)
+    out = torch.empty(R, H, device=x.device, dtype=bf)
+    for e in range(E):
+        if offs[e + 1] > offs[e]:
+            out[offs[e]:offs[e + 1]] = (inter[offs[e]:offs[e + 1]].float() @ wd[e].float()).to(bf)
+    y = torch.zeros(T, H, device=x.device).index_add_(0, tok, out.float() * s_perm[:, None])
+    # backward
+    dyp = dy[tok].float()
+    d_s = (dyp * out.float()).sum(1)                                          # [R], row order
+    d_out = dyp * s_perm[:, None]
+    del dyp
+    d_wd = torch.zeros(E, wd.shape[1], H, device=x.device)
+    d_inter = torch.empty(R, wd.shape[1], device=x.device)
+    for e in range(E):
+        if offs[e + 1] > offs[e]:
+            sl = slice(offs[e], offs[e + 1])
+            d_inter[sl] = d_out[sl] @ wd[e].float().t()
+            d_wd[e] = inter[sl].float().t() @ d_out[sl]
+    del d_out
+    sg = torch.sigmoid(gate)
+    d_gu = torch.empty(R, I2, device=x.device)
+    d_gu[:, 0::2] = d_inter * up * (sg * (1 + gate * (1 - sg)))
+    d_gu[:, 1::2] = d_inter * (gate * sg)
+    d_gu = d_gu.to(bf).float()                                                # stored in the model dtype
+    del d_inter, sg
+    d_wgu = torch.zeros(E, H, I2, device=x.device)
+    d_xp = torch.empty(R, H, device=x.device)
+    for e in range(E):
+        if offs[e + 1] > offs[e]:
+            sl = slice(offs[e], offs[e + 1])
+            d_xp[sl] = d_gu[sl] @ wgu[e].float().t()
+            d_wgu[e] = xp[sl].t() @ d_gu[sl]
+    dx_experts = torch.zeros(T, H, device=x.device).index_add_(0, tok, d_xp.to(bf).float())
+    d_scores = torch.zeros(T * K, device=x.device)
+    d_scores[cap["slot_of"].long()] = d_s                                     # slot f = k*T + t
+    return y, dx_experts, d_wgu, d_wd, d_scores.view(K, T).t().contiguous()
+
+
+def _worst_row(got, ref):
+    """largest per-row error relative to the RMS row norm of the reference (a tile written to the
+    wrong place, or not at all, shows up here however small its share of the whole tensor)"""
+    got, ref = got.float(), ref.float()
+    rms = ref.norm(dim=-1).pow(2).mean().sqrt()
+    return float(((got - ref).norm(dim=-1) / rms).max())
+
+
+@pytest.mark.parametrize("name", ["c3_qwen3_30b", "c5_stress"])
+def test_full_size_every_row_and_expert(gpu_device, name):
+    """C3 and C5 in full: EVERY row of y and dx and EVERY expert of both expert weight gradients
+    (and d_router_gate) against the reference's formulas evaluated in float32 torch ops on the device."""
+    T, H, E, K, I, bias_hot, n_hot, n_dead, _ = FULL[name]
+    print("full-size, every row and expert", name, flush=True)
+    dev = gpu_device
+    x, wr, wgu, wd, dy = device_inputs(T, H, E, I, dev, 90210, bias_hot, n_hot, n_dead)
+    layer = build_layer(torch.bfloat16, H, E, K, I, dev, loss_coeff=0.0)
+    with torch.no_grad():
+        layer.router_gate.copy_(wr)
+        layer.expert_gate_up.copy_(wgu)
+        layer.expert_down.copy_(wd)
+    layer.capture = {}
+    xg = x.clone().requires_grad_(True)
+    y = layer(xg)
+    y.backward(dy)
+    torch.cuda.synchronize()
+    cap = layer.capture
+    y_ref, dx_exp, d_wgu, d_wd, d_scores = _device_reference(x, wr, wgu, wd, dy, cap, K)
+
+    e_y, w_y = O.rel_l2(y.detach().float().cpu(), y_ref.cpu()), _worst_row(y.detach(), y_ref)
+    print(f"  y: rel-L2 {e_y:.2e}, worst row {w_y:.2e}", flush=True)
+    assert e_y <= TOL and w_y <= 5 * TOL
+    # the router's share of dx from the reference's formulas (oracle, all tokens) on the reference's score gradients
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.0)
+    counts = cap["counts"].cpu().long()
+    freq = counts.double() / counts.sum().double()
+    _, d_logits = O.router_backward(d_scores.cpu().double(), cap["probs"].cpu().double(), cap["topk_idx"].cpu().long(), freq, ocfg, T)
+    d_logits = d_logits.to(torch.bfloat16).to(dev)
+    dx_ref = dx_exp + d_logits.float() @ wr.float()
+    e_dx, w_dx = O.rel_l2(xg.grad.float().cpu(), dx_ref.cpu()), _worst_row(xg.grad, dx_ref)
+    print(f"  dx: rel-L2 {e_dx:.2e}, worst row {w_dx:.2e}", flush=True)
+    assert e_dx <= TOL and w_dx <= 5 * TOL
+    e_wr = O.rel_l2(layer.router_gate.grad.float().cpu(), (d_logits.float().t() @ x.float()).cpu())
+    print(f"  d_router_gate: rel-L2 {e_wr:.2e}", flush=True)
+    assert e_wr <= TOL
+    worst = {"gate_up": 0.0, "down": 0.0}
+    for e in range(E):
+        for nm, got, ref in (("gate_up", layer.expert_gate_up.grad[e], d_wgu[e]), ("down", layer.expert_down.grad[e], d_wd[e])):
+            if int(counts[e]) == 0:
+                assert bool((got == 0).all()), f"d_{nm}[{e}] of an expert without rows"
+                continue
+            err = float((got.float() - ref).norm() / ref.norm())
+            worst[nm] = max(worst[nm], err)
+            assert err <= TOL, f"d_{nm}[{e}]: {err:.3e}"
+            assert _worst_row(got, ref) <= 5 * TOL, f"d_{nm}[{e}]: a row is off"
+    print(f"  weight gradients, worst expert: gate_up {worst['gate_up']:.2e} down {worst['down']:.2e}", flush=True)
+
+
 def test_full_size_c4_grouped_gemms(ops, gpu_device):
     """C4: one EP rank's share of a DeepSeek-V3-like layer -- 65536 pre-assigned rows,
     32 local experts with Zipf(1.2) loads, H=7168, I=2048; forward and backward grouped GEMMs."""
@@ -225,7 +342,10 @@ def test_full_size_c4_grouped_gemms(ops, gpu_device):
     out = ops.grouped_gemm_nn(inter_s, wd, offs)
     d_inter = ops.grouped_gemm_nt(dout, wd, offs)
     d_wd = ops.grouped_gemm_wgrad(inter_s, dout, offs, E)
-    d_gu = ops.gated_act_bwd(gate_up, d_inter, row_scale=scores)
+    # the layer and bench.py run the data gradient of down with the gated-activation backward as its
+    # epilogue; the unfused pair (d_inter above, gated_act_bwd) is the cross-check
+    d_gu, parts = ops.grouped_gemm_nt_gated_bwd(dout, wd, offs, gate_up, row_scale=scores)
+    d_gu_unfused = ops.gated_act_bwd(gate_up, d_inter, row_scale=scores)
     d_xp = ops.grouped_gemm_nt(d_gu, wgu, offs)
     d_wgu = ops.grouped_gemm_wgrad(xp, d_gu, offs, E)
     torch.cuda.synchronize()
@@ -255,6 +375,17 @@ def test_full_size_c4_grouped_gemms(ops, gpu_device):
         for c in (1, 2 * I - 2):
             ref_col = xp[r0:r1].double().t() @ d_gu[r0:r1, c].double()
             assert O.rel_l2(d_wgu[e, :, c].double(), ref_col) <= TOL, f"dW_gate_up[{e}][:, {c}]"
+    # fused against unfused on ALL rows (the unfused pair rounds d_inter to the model dtype in between)
+    err = O.rel_l2(d_gu.float().cpu(), d_gu_unfused.float().cpu())
+    print(f"  fused vs unfused d_gate_up, all rows: {err:.2e}", flush=True)
+    assert err <= TOL and _worst_row(d_gu, d_gu_unfused) <= 5 * TOL
+    # the score-gradient row sums of the fused kernel: sum_i d_inter * up * act(gate), all rows
+    gu_f = gate_up.float()
+    ds_ref = (d_inter.float() * gu_f[:, 1::2] * F.silu(gu_f[:, 0::2])).sum(1)
+    err = O.rel_l2(parts.sum(0).cpu(), ds_ref.cpu())
+    print(f"  score-gradient row sums, all rows: {err:.2e}", flush=True)
+    assert err <= TOL
+    del gu_f, ds_ref, d_gu_unfused
     # rows are processed exactly once: every output row is written (no NaN / stale memory)
     for t in (gate_up, inter_s, out, d_inter, d_xp, d_wd, d_wgu):
         assert bool(torch.isfinite(t.float()).all())
