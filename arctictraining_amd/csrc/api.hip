@@ -33,7 +33,7 @@ int amoe_bf16_nt_gated_bwd(const void* dy, const int32_t* a_row_map, const void*
 int amoe_bf16_gated_bwd_parts(int I, int tile_cfg);
 int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                   int Kred, int N, int ldb, long long strideB, bool b_kc, void* workspace, size_t workspace_bytes,
-                  hipStream_t s);
+                  bool map_ready, hipStream_t s);
 int amoe_f32_wgrad(const void* A, const int32_t* a_row_map, const void* B, const int32_t* b_row_map,
                    const int32_t* offsets, void* C, int R, int E, int Kd, int N, hipStream_t s);
 int amoe_launch_gated_act_fwd(const void* gu, const float* row_scale, void* inter, int dtype, int R, int I, int act,
@@ -96,7 +96,7 @@ AMOE_EXPORT int amoe_grouped_gemm_gateup_act_fwd(const void* xp, const int32_t* 
     AMOE_REQUIRE(gate_up, AMOE_ERR_UNSUPPORTED, "%s: the f32 path needs the gate_up buffer", what);
     AMOE_REQUIRE(I % 4 == 0, AMOE_ERR_UNSUPPORTED, "%s: f32 intermediate size %d must be a multiple of 4", what, I);
     rc = amoe_f32_rows(xp, a_row_map, w_gate_up, offsets, gate_up, R, E, H, 2 * I, 2 * I, (long long)H * 2 * I, false,
-                       workspace, workspace_bytes, s);
+                       workspace, workspace_bytes, (tile_cfg & AMOE_TILE_MAP_READY) != 0, s);
     if (rc) return rc;
     return amoe_launch_gated_act_fwd(gate_up, row_scale, inter, dtype, R, I, act, s);
 }
@@ -117,7 +117,7 @@ AMOE_EXPORT int amoe_grouped_gemm_nn(const void* A, const int32_t* a_row_map, co
     if (dtype != AMOE_F32)
         return amoe_bf16_nn(A, a_row_map, B, offsets, C, R, E, Kd, N, workspace, workspace_bytes, tile_cfg, s, dtype);
     return amoe_f32_rows(A, a_row_map, B, offsets, C, R, E, Kd, N, N, (long long)Kd * N, false, workspace,
-                         workspace_bytes, s);
+                         workspace_bytes, (tile_cfg & AMOE_TILE_MAP_READY) != 0, s);
 }
 
 AMOE_EXPORT int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets,
@@ -136,7 +136,7 @@ AMOE_EXPORT int amoe_grouped_gemm_nt(const void* A, const int32_t* a_row_map, co
     if (dtype != AMOE_F32)
         return amoe_bf16_nt(A, a_row_map, B, offsets, C, R, E, Kd, N, workspace, workspace_bytes, tile_cfg, s, dtype);
     return amoe_f32_rows(A, a_row_map, B, offsets, C, R, E, /*Kred=*/N, /*N out=*/Kd, /*ldb=*/N, (long long)Kd * N, true,
-                         workspace, workspace_bytes, s);
+                         workspace, workspace_bytes, (tile_cfg & AMOE_TILE_MAP_READY) != 0, s);
 }
 
 AMOE_EXPORT int amoe_grouped_gemm_wgrad(const void* A, const int32_t* a_row_map, const void* B,

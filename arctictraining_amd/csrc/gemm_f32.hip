@@ -155,12 +155,13 @@ grouped_gemm_f32_kernel(GemmArgsF32 p)
 // rows mode: C[rows_e, :N] = A[rows_e, :Kred] @ op(B[e]);  b_kc selects B stored [N,Kred]
 int amoe_f32_rows(const void* A, const int32_t* a_row_map, const void* B, const int32_t* offsets, void* C, int R, int E,
                   int Kred, int N, int ldb, long long strideB, bool b_kc, void* workspace, size_t workspace_bytes,
-                  hipStream_t s)
+                  bool map_ready, hipStream_t s)
 {
     GemmArgsF32 a = {};
     int max_mtiles = 0;
+    // map_ready (AMOE_TILE_MAP_READY): the workspace already holds the map for these offsets, nothing is launched
     int rc = amoe_build_tile_map(offsets, R, E, BM, workspace, workspace_bytes, &a.tile_map, &a.n_mtiles, &max_mtiles, s,
-                                 /*ready=*/false);
+                                 map_ready);
     if (rc) return rc;
     a.A = (const float*)A;
     a.B = (const float*)B;

@@ -9,7 +9,6 @@ The whole routed-expert computation is one torch.autograd.Function whose forward
 backward call the kernels stage by stage with no host synchronisation.
 """
 import contextlib
-import os
 import time
 from collections import OrderedDict, defaultdict
 from dataclasses import dataclass
@@ -41,7 +40,10 @@ class MoEConfig:
     top_k: int
     use_triton: bool = True  # accepted for compatibility; the HIP kernels are always used
     use_shared_expert: bool = False
-    use_custom_moe_kernel: bool = False  # accepted for compatibility
+    # accepted for compatibility and IGNORED: the reference's capacity-padded custom-kernel path (moe.py:140-149,
+    # 413-448) differs from its default path by design (atomic row order, no load-balance gradient, scores
+    # normalised inside the gather); this layer always computes the default path and warns once when the flag is set
+    use_custom_moe_kernel: bool = False
     enable_routing_replay: bool = False
 
 
@@ -140,7 +142,9 @@ def _dense_weight_grad(a: torch.Tensor, b: torch.Tensor, tile_cfg: int = 0, tile
 
     Few output tiles and a deep reduction over the tokens: run as a split-K on the grouped
     weight-gradient kernel -- the tokens are cut into chunks that play the role of experts,
-    C[s] = a[chunk s]^T @ b[chunk s] -- and the partial products are summed in float32."""
+    C[s] = a[chunk s]^T @ b[chunk s].  The kernel accumulates each partial product in float32 and
+    stores it in the operands' 16-bit type; the (at most 16) partials are then added in float32
+    and the sum is rounded once more."""
     T, Kd = a.shape
     N = b.shape[1]
     tiles = -(-Kd // tile) * -(-N // tile)
@@ -174,10 +178,11 @@ def _route(x, router_gate, replay, opts):
     assign = topk_idx
     if replay is not None:
         assign = replay.to(torch.int32).contiguous()
-        if os.environ.get("AMOE_CHECK_REPLAY") == "1":
+        if opts.get("check_replay", True) and not torch.cuda.is_current_stream_capturing():
             # The reference's one_hot(..., num_classes=E) raises on an expert id outside [0, E)
-            # (moe.py:374); the permutation kernels clamp such ids for memory safety instead.  This
-            # opt-in check restores the error at the price of a host synchronisation.
+            # (moe.py:374).  The same error here, at the price of one host synchronisation per replayed
+            # forward; `ArcticMoE.check_replay = False` (and a HIP graph capture, which cannot
+            # synchronise) skips it, the permutation kernels then clamp such ids for memory safety.
             bad = ((assign < 0) | (assign >= E)).any()
             if bool(bad):
                 raise RuntimeError(f"routing_replay_assignments holds expert ids outside [0, {E})")
@@ -468,6 +473,14 @@ class ArcticMoE(nn.Module):
         self.num_experts = config.num_experts
         self.top_k = config.top_k
         self.use_custom_kernel = getattr(config, "use_custom_moe_kernel", False)
+        if self.use_custom_kernel:
+            import warnings
+
+            warnings.warn(
+                "ArcticMoE: use_custom_moe_kernel=True is ignored -- the layer computes the reference's default path "
+                "(ragged rows, load-balance gradient, scores normalised in the gate), not its capacity-padded one",
+                stacklevel=2,
+            )
         if self.ep_size != 1:
             raise NotImplementedError("this build runs the expert layer on one GPU (ep_size must be 1)")
         self.is_gated = bool(getattr(config, "is_gated", True))
@@ -478,6 +491,9 @@ class ArcticMoE(nn.Module):
         self.gate_time = 0.0
         self.num_local_experts = self.num_experts // self.ep_size
         self.tile_cfg = 0  # 0 = library default tile shape; other values are for tuning
+        # replayed expert ids outside [0, E) raise like the reference's one_hot (one host synchronisation per
+        # replayed forward); False: no check, the permutation kernels clamp them
+        self.check_replay = True
         self.capture = None  # set to a dict to receive the routing intermediates of each forward
 
         dt = self.input_dtype
@@ -531,6 +547,7 @@ class ArcticMoE(nn.Module):
             ep_size=self.ep_size,
             act=self._act_code,
             tile_cfg=self.tile_cfg,
+            check_replay=self.check_replay,
             want_scores=bool(getattr(self._config, "return_router_scores", False)),
             timers=self.timers,
             capture=self.capture,

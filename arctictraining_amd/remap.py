@@ -18,7 +18,10 @@ Three storage formats of the original experts are understood:
   * the gpt-oss experts (the reference's non-list branch, utils.py:291-299): `gate_up_proj` holds
     gate and up INTERLEAVED, either as [E, 2I, H] (the reference transposes it) or already as
     [E, H, 2I]; `down_proj [E, H, I]`.  Which fused format a model uses is decided by its
-    architecture (`fused_gate_up_interleaved` of the derived config), never guessed from shapes.
+    architecture (`fused_gate_up_interleaved` of the derived config).  The orientation of an
+    interleaved `gate_up_proj` is taken from `fused_gate_up_transposed` of the model's config when it
+    is set (True: stored [E, 2I, H] and transposed on install, as the reference does); without it
+    the shape decides when it can (H != 2I), and a square tensor raises instead of being guessed.
 """
 import copy
 import re
@@ -67,12 +70,35 @@ def arctic_moe_config_from_hf(config, dtype, ep_size=1, enable_routing_replay=Fa
     ns.use_shared_expert = hasattr(config, "shared_expert_intermediate_size")
     ns.return_router_scores = arch in ("GptOssForCausalLM",)
     ns.fused_gate_up_interleaved = "GptOss" in arch  # layout of a fused experts.gate_up_proj tensor
+    ns.fused_gate_up_transposed = getattr(config, "fused_gate_up_transposed", None)  # None: decided by the shape
     ns.use_triton = False
     ns.is_gated = True
     ns.use_custom_moe_kernel = False
     ns.enable_routing_replay = enable_routing_replay
     ns.ep_size, ns.ep_rank, ns.ep_group = 1, 0, None
     return ns
+
+
+def _interleaved_is_transposed(cfg, shape, H: int, I2: int) -> bool:
+    """Whether an interleaved fused gate_up_proj of `shape` is stored [E, 2I, H] (True: transposed on
+    install, what the reference always does, utils.py:296) or already [E, H, 2I] (False)."""
+    flag = getattr(cfg, "fused_gate_up_transposed", None)
+    last = tuple(shape[-2:])
+    if flag is not None:
+        want = (I2, H) if flag else (H, I2)
+        if last != want:
+            raise ValueError(f"gate_up_proj of shape {tuple(shape)}: fused_gate_up_transposed={bool(flag)} means [E, {want[0]}, {want[1]}]")
+        return bool(flag)
+    if H == I2:
+        raise ValueError(
+            f"gate_up_proj of shape {tuple(shape)} is square (hidden == 2 * intermediate): set fused_gate_up_transposed "
+            "in the model's config (True: stored [E, 2I, H], the layout the reference transposes; False: [E, H, 2I])"
+        )
+    if last == (I2, H):
+        return True
+    if last == (H, I2):
+        return False
+    raise ValueError(f"gate_up_proj of shape {tuple(shape)} is neither [E, {I2}, {H}] nor [E, {H}, {I2}]")
 
 
 def _experts_is_a_list(experts) -> bool:
@@ -99,12 +125,10 @@ def fill_arctic_moe_from_orig_mlp(arctic_moe: ArcticMoE, orig_mlp, device) -> No
         H, I2 = arctic_moe.model_dim, 2 * arctic_moe.intermediate_dim
         if getattr(arctic_moe._config, "fused_gate_up_interleaved", False):
             # gpt-oss: gate / up already interleaved; at most a batched transpose is needed
-            if tuple(fused.shape[-2:]) == (I2, H) and H != I2:
+            if _interleaved_is_transposed(arctic_moe._config, fused.shape, H, I2):
                 arctic_moe.expert_gate_up.copy_(ops.remap_pack(fused.contiguous()))
-            elif tuple(fused.shape[-2:]) == (H, I2):
-                arctic_moe.expert_gate_up.copy_(fused)
             else:
-                raise ValueError(f"gate_up_proj of shape {tuple(fused.shape)} is neither [E, {I2}, {H}] nor [E, {H}, {I2}]")
+                arctic_moe.expert_gate_up.copy_(fused)
             arctic_moe.expert_down.copy_(ops.remap_pack(down))
             return
         if tuple(fused.shape[-2:]) != (I2, H):
@@ -141,7 +165,7 @@ def fill_orig_mlp_from_arctic_moe(orig_mlp, arctic_moe: ArcticMoE) -> None:
     elif getattr(arctic_moe._config, "fused_gate_up_interleaved", False):
         fused = experts.gate_up_proj
         H, I2 = arctic_moe.model_dim, 2 * arctic_moe.intermediate_dim
-        if tuple(fused.shape[-2:]) == (I2, H) and H != I2:
+        if _interleaved_is_transposed(arctic_moe._config, fused.shape, H, I2):
             fused.copy_(ops.remap_unpack(gate_up, two=False))
         else:
             fused.copy_(gate_up)

@@ -160,19 +160,16 @@ def test_layer_routing_replay_and_returned_scores(gpu_device):
     assert O.rel_l2(scores.cpu(), ref["scores_perm"]) <= 1e-2
     with pytest.raises(AssertionError):
         layer(x.to(gpu_device))
-    # an expert id outside [0, E): clamped by default (no host sync on the hot path); the opt-in
-    # check restores the error the reference's one_hot raises (moe.py:374)
+    # an expert id outside [0, E) raises like the reference's one_hot (moe.py:374); with the check switched
+    # off the permutation kernels clamp it (no host sync on the hot path)
     bad = replay.clone()
     bad[5, 0] = E + 3
-    import os
+    with pytest.raises(RuntimeError, match="outside"):
+        layer(x.to(gpu_device), bad.to(gpu_device))
+    layer.check_replay = False
     layer(x.to(gpu_device), bad.to(gpu_device))
     torch.cuda.synchronize()
-    os.environ["AMOE_CHECK_REPLAY"] = "1"
-    try:
-        with pytest.raises(RuntimeError, match="outside"):
-            layer(x.to(gpu_device), bad.to(gpu_device))
-    finally:
-        del os.environ["AMOE_CHECK_REPLAY"]
+    layer.check_replay = True
 
 
 @pytest.mark.parametrize(

@@ -527,6 +527,36 @@ def test_grouped_gemm_every_sliver_height(ops, gpu_device, dtype, cfg):
         assert O.rel_l2(parts.sum(0).cpu(), s64.grad) <= _pick(dtype, 5e-3, 0.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("cfg", [0, 1, 3, 5])
+def test_weight_gradient_every_edge_class(ops, gpu_device, dtype, cfg):
+    """The weight gradient's live-block dispatch: output rows (Kd) that end in every remainder class of a
+    32-row block in the last row tile, output columns (N) that leave waves of the last column tile without
+    work, experts with ragged and empty row ranges.  Per expert, so that one wrong edge tile cannot hide
+    in the norm of the whole gradient."""
+    _say("wgrad edges", dtype, cfg)
+    g = torch.Generator().manual_seed(123)
+    counts = torch.tensor([1, 31, 64, 0, 97, 300, 33])
+    E, R = len(counts), int(counts.sum())
+    cs = counts.cumsum(0)
+    offs = _offsets(counts, gpu_device)
+    d = gpu_device
+    tol = _pick(dtype, 4e-3, F32_TOL)
+    for Kd, N in ((32, 72), (96, 104), (160, 200), (288, 328)):
+        A = torch.randn(R, Kd, generator=g).to(dtype)
+        G = torch.randn(R, N, generator=g).to(dtype)
+        W = ops.grouped_gemm_wgrad(A.to(d), G.to(d), offs, E, tile_cfg=cfg).cpu()
+        start = 0
+        for e in range(E):
+            end = int(cs[e])
+            if end == start:
+                assert bool((W[e] == 0).all()), f"Kd={Kd} N={N}: expert {e} has no rows"
+            else:
+                ref = A[start:end].double().t() @ G[start:end].double()
+                assert O.rel_l2(W[e], ref) <= 2 * tol, f"Kd={Kd} N={N}: expert {e} with {end - start} rows"
+            start = end
+
+
 def test_grouped_gemm_rows_outside_groups_untouched(ops, gpu_device):
     """Rows past offsets[E] are never written (the tile map covers only routed rows)."""
     g = torch.Generator().manual_seed(5)

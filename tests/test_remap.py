@@ -333,3 +333,66 @@ def test_fused_layout_mismatch_is_an_error(gpu_device):
     model.dtype = torch.float32
     with pytest.raises(ValueError, match="interleaves"):
         remap_orig_moe_mlp_params_to_arctic_moe(model, device=gpu_device)
+
+
+def _gpt_oss_model(E, K, H, I, gate_up_param, down_w, flag=None):
+    from types import SimpleNamespace
+
+    experts = torch.nn.Module()
+    experts.gate_up_proj = torch.nn.Parameter(gate_up_param)
+    experts.down_proj = torch.nn.Parameter(down_w.clone())
+    mlp = torch.nn.Module()
+    mlp.gate = torch.nn.Linear(H, E, bias=False)
+    mlp.experts = experts
+    layer = torch.nn.Module()
+    layer.mlp = mlp
+    model = torch.nn.Module()
+    model.model = torch.nn.Module()
+    model.model.layers = torch.nn.ModuleList([layer])
+    model.config = SimpleNamespace(hidden_size=H, num_experts_per_tok=K, router_aux_loss_coef=0.0, hidden_act="silu",
+                                   intermediate_size=I, num_local_experts=E, architectures=["GptOssForCausalLM"])
+    if flag is not None:
+        model.config.fused_gate_up_transposed = flag
+    model.dtype = torch.float32
+    return model
+
+
+def test_square_interleaved_gate_up_is_not_guessed():
+    """hidden == 2 * intermediate: the shape of an interleaved gate_up_proj does not tell its orientation.
+    Without the explicit flag the hook raises (no GPU needed: the error comes before any kernel)."""
+    from arctictraining_amd.remap import remap_orig_moe_mlp_params_to_arctic_moe
+
+    E, K, H, I = 2, 1, 64, 32
+    g = torch.Generator().manual_seed(3)
+    model = _gpt_oss_model(E, K, H, I, torch.randn(E, H, 2 * I, generator=g), torch.randn(E, H, I, generator=g))
+    with pytest.raises(ValueError, match="square"):
+        remap_orig_moe_mlp_params_to_arctic_moe(model, device="cpu")
+    # a flag that contradicts an unambiguous shape is an error too
+    model = _gpt_oss_model(E, K, H, 24, torch.randn(E, H, 48, generator=g), torch.randn(E, H, 24, generator=g), flag=True)
+    with pytest.raises(ValueError, match="fused_gate_up_transposed"):
+        remap_orig_moe_mlp_params_to_arctic_moe(model, device="cpu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("transposed", [True, False])
+def test_square_interleaved_gate_up_follows_the_flag(gpu_device, transposed):
+    """hidden == 2 * intermediate with fused_gate_up_transposed set: True transposes on install (what the
+    reference always does, utils.py:296), False copies; both restore the original tensor."""
+    from arctictraining_amd.remap import remap_arctic_moe_to_orig_moe_mlp_params, remap_orig_moe_mlp_params_to_arctic_moe
+
+    E, K, H, I = 4, 2, 64, 32
+    g = torch.Generator().manual_seed(9)
+    gate_w, up_w = torch.randn(E, H, I, generator=g), torch.randn(E, H, I, generator=g)
+    interleaved = torch.stack((gate_w, up_w), dim=-1).reshape(E, H, 2 * I)
+    down_w = torch.randn(E, H, I, generator=g)
+    stored = (interleaved.transpose(1, 2) if transposed else interleaved).contiguous()
+    model = _gpt_oss_model(E, K, H, I, stored, down_w, flag=transposed).to(gpu_device)
+    model.dtype = torch.float32
+    saved = {k: v.detach().clone() for k, v in model.model.layers[0].mlp.state_dict().items()}
+    remap_orig_moe_mlp_params_to_arctic_moe(model, device=gpu_device)
+    amoe = model.model.layers[0].mlp
+    assert torch.equal(amoe.expert_gate_up.detach().cpu(), interleaved)
+    remap_arctic_moe_to_orig_moe_mlp_params(model)
+    got = model.model.layers[0].mlp.state_dict()
+    for k in saved:
+        assert torch.equal(got[k], saved[k]), k

@@ -45,6 +45,47 @@ def test_permute_plan_static_matches_workspace_variant(gpu_device):
         assert int(ref[0].sum()) == T * K and int(ref[0][5]) == 0
 
 
+def test_permute_plan_static_allocates_nothing_and_runs_under_capture(gpu_device):
+    """What the entry point is for: a call leaves the device's free memory unchanged, and a call recorded
+    into a HIP graph (after one eager warm-up call) replays to the same plan as the workspace variant."""
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(5)
+    T, K, E = 4096, 4, 32
+    assign = torch.randint(0, E, (T, K), generator=g, dtype=torch.int32).to(gpu_device)
+    scores = torch.rand(T, K, generator=g).to(gpu_device)
+    R = T * K
+    i32 = dict(dtype=torch.int32, device=gpu_device)
+    outs = [torch.full((E,), -7, **i32), torch.full((E + 1,), -7, **i32), torch.full((R,), -7, **i32),
+            torch.full((R,), -7, **i32), torch.full((T, K), -7, **i32), torch.full((R,), -7.0, device=gpu_device)]
+    args = [assign.data_ptr(), scores.data_ptr(), T, K, E] + [o.data_ptr() for o in outs]
+
+    def call(stream):
+        _lib.check(lib.amoe_permute_plan_static(*args, stream), "permute_plan_static")
+
+    call(torch.cuda.current_stream().cuda_stream)   # warm-up: the scratch address is looked up on the first call
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, "the call changed the device's free memory"
+    ref = _plan(lib, False, assign, scores, E)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        for o in outs:
+            o.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, r, o in zip(("counts", "offsets", "token_of", "slot_of", "row_of", "scores_perm"), ref, outs):
+            assert torch.equal(r, o), f"{name}, replay {rep}"
+
+
 def test_permute_plan_static_rejects_oversize(gpu_device):
     lib = _lib.load()
     p = torch.empty(16, dtype=torch.int32, device=gpu_device).data_ptr()
