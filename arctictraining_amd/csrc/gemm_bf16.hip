@@ -709,18 +709,28 @@ __device__ __forceinline__ void grouped_gemm_rows_body(const GemmArgs& p)
     // Virtual blocks b, b + grid, b + 2 grid, ...; virtual block v belongs to XCD v % 8 (the hardware deals
     // workgroups to the XCDs round-robin) and is slot (v / 8) % (gm gn) of super-tile ((v / 8) / (gm gn)) * 8
     // + v % 8: the workgroups resident on one XCD work on one super-tile of gm x gn tiles at a time (its gm A
-    // panels and gn B panels are shared in that XCD's L2) and the super-tiles rotate over the XCDs.
+    // panels and gn B panels are shared in that XCD's L2) and the super-tiles rotate over the XCDs.  Only whole
+    // groups of 8 super-tiles are dealt that way: the up to 7 left over would give some XCDs a whole super-tile
+    // (about one round of tiles) more than the others, so their tiles go to the XCDs one by one.
     const int per_super = p.gm * p.gn;
     const int n_mtiles = min(scalar_load_i32(p.n_mtiles), p.max_mtiles);
-    const int vb_total = 8 * ((((n_mtiles + p.gm - 1) / p.gm) * p.sn + 7) / 8) * per_super;
+    const int supers = ((n_mtiles + p.gm - 1) / p.gm) * p.sn;
+    const int vb_rot = (supers >> 3) * 8 * per_super;      // virtual blocks of the rotated part
+    const int vb_total = supers * per_super;
     int vb_next = blockIdx.x;
     auto advance = [&](int& pm, int& nt) -> bool {  // this workgroup's next tile; false: none is left
         while (vb_next < vb_total) {
             const int vb = vb_next;
             vb_next += gridDim.x;
-            const int xcd = vb & 7, q = vb >> 3;
-            const int sid = (q / per_super) * 8 + xcd;
-            const int w = q % per_super;
+            int sid, w;
+            if (vb < vb_rot) {
+                const int xcd = vb & 7, q = vb >> 3;
+                sid = (q / per_super) * 8 + xcd;
+                w = q % per_super;
+            } else {
+                sid = vb / per_super;
+                w = vb - sid * per_super;
+            }
             const int sm = sid / p.sn, sn_i = sid - sm * p.sn;
             pm = sm * p.gm + w / p.gn;
             nt = sn_i * p.gn + w % p.gn;
