@@ -75,15 +75,25 @@ STAMP_PATH = os.path.join(LIB_DIR, "build_commit.txt")
 
 def _stamp_commit() -> None:
     """Record which commit the library was built from next to it (the stamp travels with the built
-    library to machines that have no git history; measurements quote it)."""
+    library to machines that have no git history; measurements quote it).  Two lines: the commit of
+    the tree, and the last commit that changed a file under csrc/ (the kernels themselves: a profile
+    taken at that commit stays the profile of the library through commits that touch no kernel)."""
     try:
         root = os.path.dirname(PKG_DIR)
-        head = subprocess.run(["git", "-C", root, "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True, timeout=10)
-        dirty = subprocess.run(["git", "-C", root, "status", "--porcelain", "--untracked-files=no"], capture_output=True,
-                               text=True, timeout=10)
-        if head.returncode == 0 and head.stdout.strip():
-            with open(STAMP_PATH, "w") as fh:
-                fh.write(head.stdout.strip() + ("+uncommitted" if dirty.stdout.strip() else "") + "\n")
+
+        def git(*args):
+            r = subprocess.run(["git", "-C", root, *args], capture_output=True, text=True, timeout=10)
+            return r.stdout.strip() if r.returncode == 0 else ""
+
+        head = git("rev-parse", "--short=12", "HEAD")
+        if not head:
+            return
+        dirty = git("status", "--porcelain", "--untracked-files=no")
+        kernels = git("log", "-1", "--format=%h", "--abbrev=12", "--", "arctictraining_amd/csrc")
+        kdirty = git("status", "--porcelain", "--untracked-files=no", "--", "arctictraining_amd/csrc")
+        with open(STAMP_PATH, "w") as fh:
+            fh.write(head + ("+uncommitted" if dirty else "") + "\n")
+            fh.write("kernels " + (kernels or head) + ("+uncommitted" if kdirty else "") + "\n")
     except Exception:
         pass  # no git here: leave whatever stamp came with the tree
 

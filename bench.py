@@ -84,21 +84,37 @@ def time_op(fn, iters, torch):
     return start.elapsed_time(stop) / iters
 
 
+def _git(*args):
+    try:
+        r = subprocess.run(["git", "-C", ROOT, *args], capture_output=True, text=True, timeout=10)
+        return r.stdout.strip() if r.returncode == 0 else ""
+    except Exception:
+        return ""
+
+
+def _stamp():
+    """The two lines the library build left beside the library: tree commit, kernel commit."""
+    try:
+        with open(os.path.join(ROOT, "arctictraining_amd", "lib", "build_commit.txt")) as fh:
+            lines = fh.read().split("\n")
+    except OSError:
+        return None, None
+    head = lines[0].strip() or None
+    kern = next((l.split()[1] for l in lines[1:] if l.startswith("kernels ") and len(l.split()) > 1), None)
+    return head, kern
+
+
 def git_head():
     """The commit of the running tree: from git when the history is here, otherwise the stamp that
     the library build left beside the library it built."""
-    try:
-        out = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short=12", "HEAD"], capture_output=True, text=True,
-                             timeout=10).stdout.strip()
-        if out:
-            return out
-    except Exception:
-        pass
-    try:
-        with open(os.path.join(ROOT, "arctictraining_amd", "lib", "build_commit.txt")) as fh:
-            return fh.read().strip() or None
-    except OSError:
-        return None
+    return _git("rev-parse", "--short=12", "HEAD") or _stamp()[0]
+
+
+def kernel_commit():
+    """The last commit that changed a file under arctictraining_amd/csrc (the kernels): what a
+    profile of a kernel is a profile of.  From the library's build stamp (the library is what runs);
+    from git only when there is no stamp."""
+    return _stamp()[1] or _git("log", "-1", "--format=%h", "--abbrev=12", "--", "arctictraining_amd/csrc") or None
 
 
 def cpu_baseline(name, sample_tokens, torch):
@@ -396,6 +412,7 @@ def main():
             "kernel": dom_key, "launches_per_step": dg["members"], "bound": "mfma", "achieved": round(ach, 1),
             "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4), "traffic": traffic,
             "traffic_measured_at_commit": traffic_commit,
+            "traffic_is_of_these_kernels": traffic_commit is not None and traffic_commit == kernel_commit(),
             "avg_ms": round(avg_ms, 4), "flops_per_launch": dg["flops"] / dg["n"],
             "algorithmic_bytes_per_launch": dg["bytes"] / dg["n"],
         }
@@ -405,6 +422,7 @@ def main():
             "kernel": dom_key, "launches_per_step": dg["members"], "bound": "hbm", "achieved": round(ach, 1),
             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": traffic,
             "traffic_measured_at_commit": traffic_commit,
+            "traffic_is_of_these_kernels": traffic_commit is not None and traffic_commit == kernel_commit(),
             "avg_ms": round(avg_ms, 4), "bytes_per_launch": dg["bytes"] / dg["n"],
         }
     gemm_ms = sum(e_["ms"] for e_ in breakdown if e_["_flops"])
@@ -485,6 +503,7 @@ def main():
             "tokens": T, "hidden": H, "experts": E, "top_k": K, "intermediate": I, "tile_cfg": c,
         },
         "commit": git_head(),
+        "kernel_commit": kernel_commit(),
         "tflops": tflops,
         "frac_mfma_peak": tflops / peak,
         "grouped_gemm_tflops": gemm_flop / (gemm_ms * 1e-3) / 1e12,
@@ -492,6 +511,9 @@ def main():
         "roofline": roofline,
         "yardstick": yardstick,
         "kernels": breakdown,
+        "kernels_note": "each entry is that kernel launched on its own, back to back, on the intermediates of a real "
+                        "step (roofline.avg_ms comes from these launches); a kernel repeated back to back does not run "
+                        "at the clocks and cache state it has inside a step, so the entries do not add up to ms_per_step",
     }
     if name == "c4":
         result["config"]["note"] = "a token of this workload is one routed row (the rows arrive already dispatched)"
