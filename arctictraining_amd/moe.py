@@ -125,6 +125,21 @@ class _SmallTensorCache:
 _INDEX_CACHE = _SmallTensorCache()
 
 
+_side_streams: dict = {}
+
+
+def _side_stream(device) -> "torch.cuda.Stream":
+    """One extra stream per device (default priority) for the expert weight gradients of the
+    backward pass: they feed nothing else in the layer, and every grouped GEMM here is one
+    workgroup per compute unit that ends with part of the chip idle -- launched from a second
+    stream, the next kernel's workgroups start on the compute units as the previous kernel's leave."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    st = _side_streams.get(idx)
+    if st is None:
+        st = _side_streams[idx] = torch.cuda.Stream(device=idx)
+    return st
+
+
 def _token_offsets(T: int, parts: int, device) -> torch.Tensor:
     """int32 [parts + 1]: the T tokens cut into `parts` nearly equal consecutive chunks."""
     return _INDEX_CACHE.get(
@@ -276,6 +291,28 @@ class _ExpertLayerFn(torch.autograd.Function):
             return (None,) * 9
         dy = torch.zeros_like(x) if dy is None else dy.contiguous()
 
+        # The two expert weight gradients run on a second stream beside the chain of data gradients.
+        # Fork: the side stream sees everything the main stream has queued so far (dy, the saved
+        # tensors); join (below): the main stream waits for it before this function returns, so the
+        # tensors either stream reads outlive the kernels that read them.
+        main = side = None
+        if x.is_cuda and opts.get("overlap_weight_grads", True):
+            main, side = torch.cuda.current_stream(), _side_stream(x.device)
+            side.wait_stream(main)
+
+        def on_side(fn):
+            if side is None:
+                return fn()
+            with torch.cuda.stream(side):
+                out = fn()
+            if not torch.cuda.is_current_stream_capturing():
+                out.record_stream(main)   # allocated from the side stream's pool, consumed on the main stream
+            return out
+
+        d_w_down = None
+        if ctx.needs_input_grad[3]:
+            d_w_down = on_side(lambda: ops.grouped_gemm_wgrad(inter_s, dy, offsets, E, tile_cfg=cfg, b_row_map=token_of))
+
         # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMMs' loads
         ws = ctx.gemm_ws  # still holds the forward's tile map
         fused = x.dtype != torch.float32 and cfg in (0, 1, 2)
@@ -297,12 +334,11 @@ class _ExpertLayerFn(torch.autograd.Function):
             d_gate_up, d_scores = ops.gated_act_bwd(
                 gate_up, d_inter_s, opts["act"], row_scale=scores_perm, slot_of=slot_of, tk=(T, K)
             )
-        d_w_down = None
-        if ctx.needs_input_grad[3]:
-            d_w_down = ops.grouped_gemm_wgrad(inter_s, dy, offsets, E, tile_cfg=cfg, b_row_map=token_of)
         d_w_gate_up = None
         if ctx.needs_input_grad[2]:
-            d_w_gate_up = ops.grouped_gemm_wgrad(x, d_gate_up, offsets, E, tile_cfg=cfg, a_row_map=token_of)
+            if side is not None:
+                side.wait_stream(main)   # d_gate_up
+            d_w_gate_up = on_side(lambda: ops.grouped_gemm_wgrad(x, d_gate_up, offsets, E, tile_cfg=cfg, a_row_map=token_of))
         if ds_perm is not None:
             # gradient of the returned scores [R] (row order), taken back to the slots [T,K]
             d_scores = d_scores + ds_perm.float()[row_of.long()]
@@ -340,6 +376,8 @@ class _ExpertLayerFn(torch.autograd.Function):
                 dx_dense.addmm_(d_pre, sh_out_gate.t())
                 dx_dense += ops.grouped_gemm_nt(d_sh_gu, sh_gate_up.unsqueeze(0), all_rows, tile_cfg=cfg)
             dx = ops.gather_rows_bwd(d_xp, row_of, addend=dx_dense)
+        if side is not None:
+            main.wait_stream(side)
         return dx, d_router_gate, d_w_gate_up, d_w_down, d_sh_gate_up, d_sh_down, d_sh_out_gate, None, None
 
 
@@ -511,6 +549,8 @@ class ArcticMoE(nn.Module):
             self.shared_expert_down = nn.Parameter(torch.empty((self.intermediate_dim, self.model_dim), dtype=dt))
             self.shared_expert_output_gate = nn.Parameter(torch.empty(self.model_dim, 1, dtype=dt))
         self.enable_routing_replay = getattr(config, "enable_routing_replay", False)
+        # backward: the two expert weight gradients on a second stream (see _side_stream)
+        self.overlap_weight_grads = True
 
     def enable_wall_clock_breakdown(self):
         """activate the phase timers (moe.py:153-156)"""
@@ -548,6 +588,7 @@ class ArcticMoE(nn.Module):
             act=self._act_code,
             tile_cfg=self.tile_cfg,
             check_replay=self.check_replay,
+            overlap_weight_grads=self.overlap_weight_grads,
             want_scores=bool(getattr(self._config, "return_router_scores", False)),
             timers=self.timers,
             capture=self.capture,

@@ -175,6 +175,8 @@ def main():
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
     ap.add_argument("--tile-cfg", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--serial-weight-grads", action="store_true",
+                    help="run the expert weight gradients on the main stream (the layer's default is a second stream)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0)
     ap.add_argument("--kernel-iters", type=int, default=10)
     ap.add_argument("--no-unragged", action="store_true",
@@ -251,6 +253,7 @@ def main():
         )
         layer = ArcticMoE(cfg).to(dev)
         layer.tile_cfg = c
+        layer.overlap_weight_grads = not args.serial_weight_grads
         with torch.no_grad():
             layer.router_gate.copy_(wr)
             layer.expert_gate_up.copy_(wgu)
