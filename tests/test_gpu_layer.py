@@ -114,6 +114,37 @@ def test_layer_matches_oracle(gpu_device, name):
         assert bool((got["d_expert_gate_up"][-8:] == 0).all()) and bool((got["d_expert_down"][-8:] == 0).all())
 
 
+def test_layer_end_to_end_without_logit_handover(gpu_device):
+    """Same inputs -> same routing with nothing handed from the device to the oracle: x in {-1, 0, 1}
+    with 16 non-zeros a row and router weights in {-1/8, 0, 1/8}, so every logit is a multiple of 1/8
+    of magnitude at most 2: exact in any summation order and in bf16, and full of ties.  The oracle
+    computes its own logits (float64) and must select, count and permute exactly as the layer did."""
+    dtype, T, H, E, K, I = torch.bfloat16, 4096, 256, 64, 4, 128
+    x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=77)
+    g = torch.Generator().manual_seed(78)
+    xs = torch.zeros(T, H)
+    cols = torch.rand(T, H, generator=g).argsort(dim=1)[:, :16]
+    xs.scatter_(1, cols, torch.randint(0, 2, (T, 16), generator=g).float() * 2 - 1)
+    x = xs.to(dtype)
+    wr = (torch.randint(-1, 2, (E, H), generator=g).float() / 8).to(dtype)
+    layer = build_layer(dtype, H, E, K, I, gpu_device)
+    got = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+    ocfg = O.OracleConfig(model_dim=H, intermediate_dim=I, num_experts=E, top_k=K, loss_coeff=0.001)
+    ref = O.forward_backward(x, wr, wgu, wd, dy, ocfg, compute_dtype=torch.float64)
+    cap = got["cap"]
+    assert torch.equal(cap["logits"].double(), ref["logits"].double()), "the logits are exact on both sides"
+    # ties: most tokens have a repeated value among their top logits, so the order of equal values matters
+    top = ref["logits"].double().topk(K + 1, dim=1).values
+    assert float((top[:, :-1] == top[:, 1:]).any(dim=1).float().mean()) > 0.5
+    assert torch.equal(cap["topk_idx"].long(), ref["topk_idx"]), "top-k indices"
+    assert torch.equal(cap["counts"].long(), ref["counts"]), "per-expert counts"
+    assert torch.equal(cap["slot_of"].long(), ref["perm"]), "permutation order"
+    assert torch.equal(cap["token_of"].long(), ref["token_ids"]), "token ids"
+    for k in ("y", "dx", "d_router_gate", "d_expert_gate_up", "d_expert_down"):
+        err = O.rel_l2(got[k], ref[k])
+        assert err <= TOL[dtype], f"{k}: rel-L2 {err:.3e}"
+
+
 def test_layer_3d_input_and_no_normalisation(gpu_device):
     dtype, T, H, E, K, I = torch.bfloat16, 512, 128, 16, 4, 64
     x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=5)
@@ -282,6 +313,25 @@ def test_layer_is_deterministic(gpu_device):
     b = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
     for k in ("y", "dx", "d_router_gate", "d_expert_gate_up", "d_expert_down"):
         assert torch.equal(a[k], b[k]), f"{k} differs between two identical runs"
+
+
+def test_weight_gradients_on_the_second_stream_match_the_serial_order(gpu_device):
+    """The backward runs the two expert weight gradients on a second stream (layer.overlap_weight_grads,
+    on by default).  Every gradient must be bit-identical to the run with everything on one stream, over
+    several steps in a row (a missing wait between the streams shows up as a stale or half-written tensor)."""
+    dtype, T, H, E, K, I = torch.bfloat16, 4096, 256, 32, 4, 384
+    layer = build_layer(dtype, H, E, K, I, gpu_device)
+    assert layer.overlap_weight_grads is True
+    keys = ("y", "dx", "d_router_gate", "d_expert_gate_up", "d_expert_down")
+    for seed in (21, 22, 23):
+        x, wr, wgu, wd, dy = O.make_inputs(T, H, E, K, I, dtype, seed=seed)
+        layer.overlap_weight_grads = False
+        serial = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+        layer.overlap_weight_grads = True
+        for rep in range(3):
+            both = run_layer(layer, x, wr, wgu, wd, dy, gpu_device)
+            for k in keys:
+                assert torch.equal(serial[k], both[k]), f"{k}, seed {seed}, repetition {rep}"
 
 
 def test_module_surface(gpu_device):
