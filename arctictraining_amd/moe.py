@@ -309,10 +309,6 @@ class _ExpertLayerFn(torch.autograd.Function):
                 out.record_stream(main)   # allocated from the side stream's pool, consumed on the main stream
             return out
 
-        d_w_down = None
-        if ctx.needs_input_grad[3]:
-            d_w_down = on_side(lambda: ops.grouped_gemm_wgrad(inter_s, dy, offsets, E, tile_cfg=cfg, b_row_map=token_of))
-
         # d(out_s)[r] = dy[token_of[r]]: the rows of dy are gathered inside the GEMMs' loads
         ws = ctx.gemm_ws  # still holds the forward's tile map
         fused = x.dtype != torch.float32 and cfg in (0, 1, 2)
@@ -334,6 +330,11 @@ class _ExpertLayerFn(torch.autograd.Function):
             d_gate_up, d_scores = ops.gated_act_bwd(
                 gate_up, d_inter_s, opts["act"], row_scale=scores_perm, slot_of=slot_of, tk=(T, K)
             )
+        # (queued after the data gradient above, which it does not depend on: its workgroups take the
+        # compute units as that kernel's last tiles finish)
+        d_w_down = None
+        if ctx.needs_input_grad[3]:
+            d_w_down = on_side(lambda: ops.grouped_gemm_wgrad(inter_s, dy, offsets, E, tile_cfg=cfg, b_row_map=token_of))
         d_w_gate_up = None
         if ctx.needs_input_grad[2]:
             if side is not None:
