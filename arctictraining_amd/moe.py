@@ -497,6 +497,13 @@ class ArcticMoE(nn.Module):
     Args:
         config: MoEConfig (or any object with the same attributes; the reference passes a
                 SimpleNamespace, utils.py:107-161)
+
+    Attributes beyond the reference's, all optional:
+        tile_cfg: tile shape of the grouped GEMMs (0 = the library's default; 1, 2, 3, 5 for tuning)
+        check_replay: raise on a replayed expert id outside [0, E), as the reference's one_hot does
+                (one host synchronisation per replayed forward; skipped under graph capture)
+        overlap_weight_grads: run the two expert weight gradients of the backward on a second stream
+        capture: a dict that receives the routing intermediates of each forward (tests)
     """
 
     def __init__(self, config):
